@@ -152,7 +152,9 @@ class CacheManager:
         if src in self._where:
             g, i = self._where[src]
             grp = self.groups[g]
-            return LayerCacheView(g, self.page_size, grp.k[i], grp.v[i], src == pos, state)
+            # a need whose values are its keys has no value pool
+            v = grp.v[i] if grp.need.value_width > 0 else None
+            return LayerCacheView(g, self.page_size, grp.k[i], v, src == pos, state)
         return LayerCacheView(-1, self.page_size, None, None, src == pos, state)
 
     # ------------------------------------------------------------------ requests
@@ -251,7 +253,8 @@ class CacheManager:
                 from .. import ops
                 idx = torch.tensor(pages, dtype=torch.int32, device=self.device)
                 ops.poison_pages(grp.k, idx)
-                ops.poison_pages(grp.v, idx)
+                if grp.v.numel() > 0:
+                    ops.poison_pages(grp.v, idx)
             else:
                 idx = torch.tensor(pages, dtype=torch.long, device=self.device)
                 grp.k[:, idx] = float("nan")

@@ -60,6 +60,9 @@ def entry_for(config: dict) -> ArchitectureEntry:
     """`decoder_family.zig:267-281`: a missing ``model_type`` and a non-string one are errors
     of their own; an unknown one is UnsupportedModelType."""
     archs = config.get("architectures", [])
+    one = config.get("architecture")            # some families name themselves in one string
+    if isinstance(one, str) and one in _BY_NAME:
+        return _BY_NAME[one]
     if isinstance(archs, list):
         for a in archs:
             if isinstance(a, str) and a in _BY_NAME:

@@ -20,6 +20,18 @@ class RmsNormSpec:
 
 
 @dataclass(frozen=True)
+class LayerNormSpec:
+    """n = (x - mean) / sqrt(mean((x - mean)^2) + eps) * w + b over ``width`` elements;
+    ``centred`` False leaves the mean in (an RMS norm with a bias).  The gain is the tensor
+    ``prefix + weight_name``, the bias ``prefix + bias_name`` (None: no bias)."""
+    width: int
+    eps: float
+    centred: bool = True
+    weight_name: str = "weight"
+    bias_name: Optional[str] = "bias"
+
+
+@dataclass(frozen=True)
 class RotaryHalfSplitSpec:
     """Rotation of the pairs (i, i + head_dim/2) by position * theta^(-2i/head_dim)."""
     head_dim: int
@@ -47,6 +59,60 @@ class GqaAttentionSpec:
 
 
 @dataclass(frozen=True)
+class TiedKeyValueAttentionSpec:
+    """Causal grouped-query attention whose values are its keys as projected (there is no
+    value projection, and the cache holds keys only), without a position encoding.
+    ``window`` as in ``GqaAttentionSpec``.  ``sink``: the soft-max's denominator holds one more
+    term of score 0 that brings no value.  ``output_gate``: the concatenated heads are
+    multiplied by sigmoid(W_g h), h being the input the projections read, before the output
+    projection.  The ``*_name`` fields are the tensor names below the mixer's prefix."""
+    hidden_size: int
+    n_heads: int
+    n_kv_heads: int
+    head_dim: int
+    scale: Optional[float] = None          # None: 1/sqrt(head_dim)
+    window: Optional[int] = None
+    sink: bool = False
+    output_gate: bool = False
+    q_name: str = "q_proj.weight"
+    k_name: str = "k_proj.weight"
+    gate_name: str = "g_proj.weight"
+    o_name: str = "o_proj.weight"
+
+
+@dataclass(frozen=True)
+class GatedExpertSpec:
+    """down(act(gate(x), up(x))) with g = min(gate, limit), u = clamp(up, -limit, limit)
+    (``limit`` None: neither is clamped) and act = g * sigmoid(alpha * g) * (u + shift)."""
+    intermediate_size: int
+    limit: Optional[float] = None
+    alpha: float = 1.0
+    shift: float = 0.0
+
+
+@dataclass(frozen=True)
+class MoeSpec:
+    """Of ``n_experts`` experts every token uses the ``top_k`` whose router logits
+    z = W_r x (+ b_r) are largest, weighted by the soft-max over those logits alone; an
+    optional ``shared`` expert runs for every token with weight 1.  Tensor names below the
+    part's prefix: the router's matrix and bias, ``expert_prefix.format(e)`` and
+    ``shared_prefix`` followed by the three matrices' names."""
+    hidden_size: int
+    n_experts: int
+    top_k: int
+    expert: GatedExpertSpec
+    shared: Optional[GatedExpertSpec] = None
+    router_bias: bool = False
+    router_name: str = "gate.weight"
+    router_bias_name: str = "gate.bias"
+    expert_prefix: str = "experts.{}."
+    shared_prefix: str = "shared_expert."
+    gate_name: str = "gate_proj.weight"
+    up_name: str = "up_proj.weight"
+    down_name: str = "down_proj.weight"
+
+
+@dataclass(frozen=True)
 class SwiGluSpec:
     """down(silu(gate(x)) * up(x))."""
     hidden_size: int
@@ -65,6 +131,25 @@ class PreNormBlockSpec:
     ff_prefix: str = "mlp."
     mixer_norm_prefix: str = "input_layernorm."
     ff_norm_prefix: str = "post_attention_layernorm."
+
+
+@dataclass(frozen=True)
+class SandwichNormBlockSpec:
+    """x += post1(mixer(norm1(x))); x += post2(ff(norm2(x))): every sublayer has a norm before
+    it and one after it, ahead of the residual sum.  ``feed_forward`` None: the layer is its
+    mixer alone (and declares neither ``ff_norm`` nor ``ff_post_norm``)."""
+    mixer: object
+    feed_forward: Optional[object]
+    mixer_norm: object
+    mixer_post_norm: object
+    ff_norm: Optional[object] = None
+    ff_post_norm: Optional[object] = None
+    mixer_prefix: str = "self_attn."
+    ff_prefix: str = "mlp."
+    mixer_norm_prefix: str = "input_layernorm."
+    mixer_post_norm_prefix: str = "post_attention_layernorm."
+    ff_norm_prefix: str = "pre_feedforward_layernorm."
+    ff_post_norm_prefix: str = "post_feedforward_layernorm."
 
 
 @dataclass(frozen=True)
@@ -96,3 +181,6 @@ class ModelSpec:
     embedding_multiplier: float = 1.0       # the embedding row times this enters the stream
     logit_scale: float = 1.0                # logits = head(x) * logit_scale ...
     logit_softcap: Optional[float] = None   # ... then cap * tanh(logits / cap) if given
+    # a learned position table [max_positions, hidden]: its row at a token's position is added
+    # to the embedding row (not scaled); None: positions enter through the mixers only
+    position_table_name: Optional[str] = None

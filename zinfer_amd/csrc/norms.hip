@@ -1,0 +1,155 @@
+// Norms over the rows of a float32 matrix, with a gain and an optional bias, that either
+// store their result (float32 or bfloat16) or add it to a float32 destination:
+//
+//   centred:      n_i = (x_i - mean) / sqrt(mean((x - mean)^2) + eps) * w_i + b_i   (layer norm)
+//   not centred:  n_i = x_i / sqrt(mean(x^2) + eps) * w_i (+ b_i)                   (RMS norm)
+//
+// All arithmetic is 32-bit.  The mean is taken first and the variance from the deviations
+// (two passes over a row that is kept in registers), never as mean(x^2) - mean^2.  One
+// workgroup per row; its result depends on that row alone.
+#include "zf_common.h"
+
+template <typename TO, bool ADD>
+__device__ __forceinline__ void norm_store(TO* o, float v) {
+  if constexpr (ADD) {
+    *o = (TO)(*o + v);      // ADD is only instantiated with TO = float
+  } else {
+    store_from_float<TO>(o, v);
+  }
+}
+
+// any width: the row is read three times
+template <typename TO, bool ADD>
+__global__ __launch_bounds__(256) void norm_rows_kernel(const float* __restrict__ x,
+                                                        const float* __restrict__ gain,
+                                                        const float* __restrict__ bias,
+                                                        TO* __restrict__ out, int W, float eps,
+                                                        int centred) {
+  __shared__ float red[16];
+  const float* row = x + (size_t)blockIdx.x * W;
+  TO* o = out + (size_t)blockIdx.x * W;
+  float mean = 0.f;
+  if (centred) {
+    float s = 0.f;
+    for (int i = threadIdx.x; i < W; i += blockDim.x) s += row[i];
+    mean = block_sum(s, red) / (float)W;
+  }
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    const float d = row[i] - mean;
+    ss += d * d;
+  }
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)W + eps);
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    float v = (row[i] - mean) * inv * gain[i];
+    if (bias != nullptr) v += bias[i];
+    norm_store<TO, ADD>(o + i, v);
+  }
+}
+
+// widths that are a multiple of 4 up to 8192: a thread keeps its part of the row (at most 8
+// float4) in registers, so the row is read once
+template <typename TO, bool ADD>
+__global__ __launch_bounds__(256) void norm_rows_vec_kernel(const float* __restrict__ x,
+                                                            const float* __restrict__ gain,
+                                                            const float* __restrict__ bias,
+                                                            TO* __restrict__ out, int W,
+                                                            float eps, int centred) {
+  __shared__ float red[16];
+  const float4* row = (const float4*)(x + (size_t)blockIdx.x * W);
+  TO* o = out + (size_t)blockIdx.x * W;
+  const int n4 = W / 4;
+  float4 v[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int c = threadIdx.x + i * 256;
+    v[i] = c < n4 ? row[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  float mean = 0.f;
+  if (centred) {
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+    mean = block_sum(s, red) / (float)W;
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int c = threadIdx.x + i * 256;
+    if (c < n4) {
+      v[i].x -= mean; v[i].y -= mean; v[i].z -= mean; v[i].w -= mean;
+      ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+    }
+  }
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)W + eps);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int c = threadIdx.x + i * 256;
+    if (c < n4) {
+      const float4 g = ((const float4*)gain)[c];
+      float4 b = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (bias != nullptr) b = ((const float4*)bias)[c];
+      norm_store<TO, ADD>(o + 4 * c + 0, v[i].x * inv * g.x + b.x);
+      norm_store<TO, ADD>(o + 4 * c + 1, v[i].y * inv * g.y + b.y);
+      norm_store<TO, ADD>(o + 4 * c + 2, v[i].z * inv * g.z + b.z);
+      norm_store<TO, ADD>(o + 4 * c + 3, v[i].w * inv * g.w + b.w);
+    }
+  }
+}
+
+template <typename TO, bool ADD>
+static void launch_norm_rows(const float* x, const float* gain, const float* bias, void* out,
+                             int T, int W, float eps, int centred, hipStream_t stream) {
+  if (W % 4 == 0 && W <= 8192)
+    hipLaunchKernelGGL((norm_rows_vec_kernel<TO, ADD>), dim3(T), dim3(256), 0, stream, x, gain,
+                       bias, (TO*)out, W, eps, centred);
+  else
+    hipLaunchKernelGGL((norm_rows_kernel<TO, ADD>), dim3(T), dim3(256), 0, stream, x, gain, bias,
+                       (TO*)out, W, eps, centred);
+}
+
+// out = norm(x) (add == 0) or out += norm(x) (add != 0, out float32); bias may be null
+extern "C" int zf_norm_rows(const float* x, const float* gain, const float* bias, void* out,
+                            int out_dtype, int T, int W, float eps, int centred, int add,
+                            hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (W <= 0 || (add && out_dtype != ZF_F32)) return -2;
+  if (add)
+    launch_norm_rows<float, true>(x, gain, bias, out, T, W, eps, centred, stream);
+  else if (out_dtype == ZF_F32)
+    launch_norm_rows<float, false>(x, gain, bias, out, T, W, eps, centred, stream);
+  else
+    launch_norm_rows<bf16_t, false>(x, gain, bias, out, T, W, eps, centred, stream);
+  ZF_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------- embedding plus a learned position
+// x[t, :] = E[id[t], :] * scale + P[position[t], :], widened to float32
+template <typename TW>
+__global__ void embed_position_kernel(const TW* __restrict__ table, const int* __restrict__ ids,
+                                      const TW* __restrict__ pos_table,
+                                      const int* __restrict__ positions, float* __restrict__ out,
+                                      int H, float scale) {
+  const int t = blockIdx.x;
+  const TW* row = table + (size_t)ids[t] * H;
+  const TW* prow = pos_table + (size_t)positions[t] * H;
+  float* o = out + (size_t)t * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x)
+    o[i] = load_as_float<TW>(row + i) * scale + load_as_float<TW>(prow + i);
+}
+
+extern "C" int zf_embed_position(const void* table, const void* pos_table, int table_dtype,
+                                 const int* ids, const int* positions, float* out, int T, int H,
+                                 float scale, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (table_dtype == ZF_F32)
+    hipLaunchKernelGGL(embed_position_kernel<float>, dim3(T), dim3(256), 0, stream,
+                       (const float*)table, ids, (const float*)pos_table, positions, out, H, scale);
+  else
+    hipLaunchKernelGGL(embed_position_kernel<bf16_t>, dim3(T), dim3(256), 0, stream,
+                       (const bf16_t*)table, ids, (const bf16_t*)pos_table, positions, out, H,
+                       scale);
+  ZF_CHECK_LAUNCH();
+}

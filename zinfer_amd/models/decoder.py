@@ -25,7 +25,9 @@ class DecoderModel:
         self.graph_safe = self.final_norm.graph_safe and all(b.graph_safe for b in self.blocks)
         # embedding, row gather and head are the model's own launches
         self.kernel_modules = tuple(sorted(
-            {"elementwise", "gemm"} | {m for b in self.blocks for m in b.kernel_modules}))
+            {"elementwise", "gemm"} | ({"norms"} if spec.position_table_name is not None else set())
+            | set(self.final_norm.kernel_modules)
+            | {m for b in self.blocks for m in b.kernel_modules}))
         for pos, e in enumerate(spec.schedule):
             if not (0 <= e.layer < len(self.blocks)):
                 raise ConfigError(f"schedule[{pos}] names layer {e.layer} of {len(self.blocks)}")
@@ -42,6 +44,8 @@ class DecoderModel:
     def declare(self) -> Dict[str, TensorDecl]:
         s = self.spec
         d: Dict[str, TensorDecl] = {s.embed_name: TensorDecl((s.vocab_size, s.hidden_size))}
+        if s.position_table_name is not None:
+            d[s.position_table_name] = TensorDecl((s.max_positions, s.hidden_size))
         for b in self.blocks:
             d.update(b.declare())
         d.update(self.final_norm.declare())
@@ -52,6 +56,12 @@ class DecoderModel:
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         s = self.spec
         self.embedding = place_matrix(tensors[s.embed_name], self.ctx)
+        self.position_table = None
+        if s.position_table_name is not None:
+            table = tensors[s.position_table_name]
+            if table.dtype != tensors[s.embed_name].dtype:
+                table = table.to(tensors[s.embed_name].dtype)
+            self.position_table = place_matrix(table, self.ctx)
         for b in self.blocks:
             b.bind(tensors)
         self.final_norm.bind(tensors)
@@ -90,7 +100,11 @@ class DecoderModel:
         s = self.spec
         T = step.n_tokens
         x = step.scratch("residual", (T, s.hidden_size), torch.float32)
-        ops.embed(self.embedding, step.token_ids, x, float(s.embedding_multiplier))
+        if self.position_table is not None:
+            ops.embed_position(self.embedding, step.token_ids, self.position_table,
+                               step.positions, x, float(s.embedding_multiplier))
+        else:
+            ops.embed(self.embedding, step.token_ids, x, float(s.embedding_multiplier))
         step.norm_ready = None
         for pos, e in enumerate(s.schedule):
             # the norm that reads the stream after this block: the next block's first, or the

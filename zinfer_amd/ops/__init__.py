@@ -1401,6 +1401,199 @@ def paged_attention(q, k_pool, v_pool, block_table, q_start, ctx_len, seq_index,
         "paged_attention")
 
 
+# ------------------------------------------------------------------------- norms with a bias
+@_launches("norm_rope_write")
+def norm_rows(x: torch.Tensor, gain: torch.Tensor, bias: Optional[torch.Tensor], eps: float,
+              out: torch.Tensor, centred: bool = True, add: bool = False) -> None:
+    """Row by row over float32 ``x`` [T, W], all in 32-bit: centred,
+    n = (x - mean) / sqrt(mean((x - mean)^2) + eps) * gain + bias (a layer norm); not centred,
+    n = x / sqrt(mean(x^2) + eps) * gain (+ bias).  ``out`` = n (float32 or bfloat16), or with
+    ``add`` out += n (float32: a branch's normed output joins the residual stream)."""
+    _need_gpu(x, gain, bias, out)
+    T, W = x.shape
+    if x.dtype != torch.float32 or gain.dtype != torch.float32 or gain.shape != (W,) \
+            or out.shape != x.shape or (bias is not None and (bias.dtype != torch.float32
+                                                              or bias.shape != (W,))) \
+            or (add and out.dtype != torch.float32):
+        raise KernelUnavailable(f"norm_rows: x {tuple(x.shape)} {x.dtype}, gain "
+                                f"{tuple(gain.shape)} {gain.dtype}, out {tuple(out.shape)} "
+                                f"{out.dtype} (float32 when added to)")
+    lib = build.load("norms")
+    _check(lib.zf_norm_rows(_ptr(x), _ptr(gain), _ptr(bias), _ptr(out), _dt(out), T, W,
+                            ctypes.c_float(eps), 1 if centred else 0, 1 if add else 0,
+                            _stream()), "norm_rows")
+
+
+@_launches("other")
+def embed_position(table: torch.Tensor, ids: torch.Tensor, pos_table: torch.Tensor,
+                   positions: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:
+    """out[t, :] = table[ids[t], :] * scale + pos_table[positions[t], :], in float32."""
+    _need_gpu(table, ids, pos_table, positions, out)
+    _i32(ids, "ids")
+    _i32(positions, "positions")
+    T, H = out.shape
+    if table.shape[1] != H or pos_table.shape[1] != H or table.dtype != pos_table.dtype \
+            or ids.shape[0] != T or positions.shape[0] != T or out.dtype != torch.float32:
+        raise KernelUnavailable(f"embed_position: table {tuple(table.shape)} {table.dtype}, "
+                                f"positions' table {tuple(pos_table.shape)} {pos_table.dtype}, "
+                                f"out {tuple(out.shape)} {out.dtype}")
+    lib = build.load("norms")
+    _check(lib.zf_embed_position(_ptr(table), _ptr(pos_table), _dt(table), _ptr(ids),
+                                 _ptr(positions), _ptr(out), T, H, ctypes.c_float(scale),
+                                 _stream()), "embed_position")
+
+
+# ------------------------------------------------------------------------- attention whose values are its keys
+def _columns(t: torch.Tensor, what: str) -> int:
+    """Row stride (in elements) of a 2-D tensor whose rows are contiguous: a slice of columns
+    of a wider product."""
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise KernelUnavailable(f"{what} must be a matrix with contiguous rows")
+    return t.stride(0)
+
+
+@_launches("norm_rope_write")
+def kv_rows_write(rows: torch.Tensor, slot_mapping: torch.Tensor, k_pool: torch.Tensor,
+                  n_kv_heads: int, head_dim: int, page_size: int) -> None:
+    """rows [T, nKV * hd] (contiguous rows, any row stride: columns of a wider product) go
+    into the pool laid out [page, kv head, row, hd] at ``slot_mapping``."""
+    for t in (rows, slot_mapping, k_pool):
+        if not t.is_cuda:
+            raise KernelUnavailable("the HIP kernels run on GPU tensors only")
+    _i32(slot_mapping, "slot_mapping")
+    T = rows.shape[0]
+    stride = _columns(rows, "kv_rows_write: rows")
+    if rows.shape[1] != n_kv_heads * head_dim or rows.dtype != k_pool.dtype \
+            or slot_mapping.shape[0] != T or not k_pool.is_contiguous() \
+            or k_pool.numel() % (n_kv_heads * head_dim * page_size) != 0:
+        raise KernelUnavailable(f"kv_rows_write: rows {tuple(rows.shape)} {rows.dtype} for "
+                                f"{n_kv_heads} heads of {head_dim}, pool {k_pool.dtype}")
+    lib = build.load("sink_attention")
+    _check(lib.zf_kv_rows_write(_ptr(rows), _dt(rows), ctypes.c_longlong(stride), 0,
+                                _ptr(slot_mapping), _ptr(k_pool), T, n_kv_heads, head_dim,
+                                page_size, _stream()), "kv_rows_write")
+
+
+@_launches("attention")
+def shared_kv_attention(q: torch.Tensor, gate: Optional[torch.Tensor], k_pool: torch.Tensor,
+                        block_table, q_start, ctx_len, seq_index, out: torch.Tensor,
+                        scale: float, window: int, sink: bool, n_heads: int, n_kv_heads: int,
+                        head_dim: int, page_size: int, max_ctx_len: int) -> None:
+    """Causal grouped-query attention whose values are the keys, over a paged pool of keys
+    [page, kv head, row, hd].  Token t of sequence s = seq_index[t] has position ctx_len[s] -
+    q_len[s] + (t - q_start[s]) and reads the positions up to its own (the last ``window`` of
+    them if window > 0).  ``sink``: the soft-max's denominator holds one more term, exp(0).
+    ``gate`` [T, nH * hd]: the output is multiplied by sigmoid(gate).  ``q`` and ``gate`` may
+    be column slices of a wider product.  Scores and weights are 32-bit in both dtypes."""
+    for t in (q, gate, k_pool, block_table, q_start, ctx_len, seq_index, out):
+        if t is not None and not t.is_cuda:
+            raise KernelUnavailable("the HIP kernels run on GPU tensors only")
+    T = q.shape[0]
+    qs = _columns(q, "shared_kv_attention: q")
+    gs = _columns(gate, "shared_kv_attention: gate") if gate is not None else 0
+    if q.shape[1] != n_heads * head_dim or out.shape != (T, n_heads * head_dim) \
+            or not out.is_contiguous() or out.dtype != q.dtype or k_pool.dtype != q.dtype \
+            or (gate is not None and (gate.shape != q.shape or gate.dtype != q.dtype)):
+        raise KernelUnavailable("shared_kv_attention: q, gate and out must be [T, nH * hd] of "
+                                "the pool's dtype")
+    for t, name in ((block_table, "block_table"), (q_start, "q_start"), (ctx_len, "ctx_len"),
+                    (seq_index, "seq_index")):
+        _i32(t, name)
+    if n_kv_heads <= 0 or n_heads % n_kv_heads != 0:
+        raise KernelUnavailable("shared_kv_attention: InvalidGrouping")
+    if not 0 < head_dim <= MAX_HEAD_DIM:
+        raise KernelUnavailable(f"shared_kv_attention: head_dim {head_dim} is not in 1.."
+                                f"{MAX_HEAD_DIM}")
+    if max_ctx_len > block_table.shape[1] * page_size:
+        raise KernelUnavailable("shared_kv_attention: block table shorter than the context")
+    n_seqs = ctx_len.shape[0]
+    if q_start.shape[0] != n_seqs + 1 or block_table.shape[0] != n_seqs \
+            or seq_index.shape[0] != T or not block_table.is_contiguous():
+        raise KernelUnavailable("shared_kv_attention: per-sequence arrays disagree in length")
+    lib = build.load("sink_attention")
+    _check(lib.zf_shared_kv_attention(
+        _ptr(q), ctypes.c_longlong(qs), _ptr(gate), ctypes.c_longlong(gs), _ptr(k_pool), _dt(q),
+        _ptr(block_table), _ptr(q_start), _ptr(ctx_len), _ptr(seq_index), _ptr(out),
+        ctypes.c_float(scale), int(window), 1 if sink else 0, T, n_heads, n_kv_heads, head_dim,
+        page_size, block_table.shape[1], _stream()), "shared_kv_attention")
+
+
+# ------------------------------------------------------------------------- mixture of experts
+MOE_MAX_EXPERTS = 1024
+
+
+@_launches("other")
+def moe_route(h: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor],
+              ids: torch.Tensor, weights: torch.Tensor) -> None:
+    """Per row of ``h`` [T, W]: z = router h + bias in 32-bit (router float32 [E, W]); ``ids``
+    [T, top] int32 receives the ``top`` largest (the lower index wins a tie), ``weights``
+    [T, top] float32 the soft-max over those alone."""
+    _need_gpu(h, router, bias, ids, weights)
+    _i32(ids, "ids")
+    T, W = h.shape
+    E = router.shape[0]
+    top = ids.shape[1] if ids.dim() == 2 else 0
+    if router.dtype != torch.float32 or router.shape != (E, W) or ids.shape != (T, top) \
+            or weights.shape != (T, top) or weights.dtype != torch.float32 \
+            or not 0 < top <= E <= MOE_MAX_EXPERTS \
+            or (bias is not None and (bias.dtype != torch.float32 or bias.shape != (E,))):
+        raise KernelUnavailable(f"moe_route: h {tuple(h.shape)}, router {tuple(router.shape)} "
+                                f"{router.dtype}, ids {tuple(ids.shape)}, at most "
+                                f"{MOE_MAX_EXPERTS} experts")
+    lib = build.load("moe")
+    _check(lib.zf_moe_route(_ptr(h), _dt(h), _ptr(router), _ptr(bias), _ptr(ids), _ptr(weights),
+                            T, W, E, top, _stream()), "moe_route")
+
+
+@_launches("products")
+def moe_gate_up(h: torch.Tensor, gate_up: torch.Tensor, ids: Optional[torch.Tensor],
+                y: torch.Tensor, limit: float, alpha: float, shift: float) -> None:
+    """y[t, s, :] = act(expert ids[t, s] of ``gate_up`` [E, 2 ff, W] applied to h[t]) with
+    g = min(gate, limit), u = clamp(up, -limit, limit) (no clamp if limit <= 0) and
+    act = g * sigmoid(alpha g) * (u + shift).  ``ids`` None: expert 0 for every token."""
+    _need_gpu(h, gate_up, ids, y)
+    T, W = h.shape
+    if y.dim() != 3 or gate_up.dim() != 3:
+        raise KernelUnavailable("moe_gate_up: y [T, slots, ff], gate_up [E, 2 ff, W]")
+    slots, ff = y.shape[1], y.shape[2]
+    if ids is not None:
+        _i32(ids, "ids")
+    if y.shape[0] != T or gate_up.shape[1:] != (2 * ff, W) or gate_up.dtype != h.dtype \
+            or y.dtype != h.dtype or (ids is not None and ids.shape != (T, slots)) \
+            or (ids is None and gate_up.shape[0] != 1) or W > 16384:
+        raise KernelUnavailable(f"moe_gate_up: h {tuple(h.shape)} {h.dtype}, gate_up "
+                                f"{tuple(gate_up.shape)} {gate_up.dtype}, y {tuple(y.shape)}")
+    lib = build.load("moe")
+    _check(lib.zf_moe_gate_up(_ptr(h), _ptr(gate_up), _dt(h), _ptr(ids), _ptr(y), T, W, ff,
+                              slots, ctypes.c_float(limit), ctypes.c_float(alpha),
+                              ctypes.c_float(shift), _stream()), "moe_gate_up")
+
+
+@_launches("products")
+def moe_down(y: torch.Tensor, down: torch.Tensor, ids: Optional[torch.Tensor],
+             weights: Optional[torch.Tensor], out: torch.Tensor, add: bool = False) -> None:
+    """out[t] (=, or with ``add`` +=) sum over s of weights[t, s] * down[ids[t, s]] y[t, s], in
+    slot order and 32-bit; ``down`` [E, W, ff], ``out`` float32 [T, W].  ``ids`` None: expert
+    0; ``weights`` None: 1."""
+    _need_gpu(y, down, ids, weights, out)
+    if y.dim() != 3 or down.dim() != 3:
+        raise KernelUnavailable("moe_down: y [T, slots, ff], down [E, W, ff]")
+    T, slots, ff = y.shape
+    W = down.shape[1]
+    if ids is not None:
+        _i32(ids, "ids")
+    if down.shape[2] != ff or down.dtype != y.dtype or out.shape != (T, W) \
+            or out.dtype != torch.float32 or (ids is not None and ids.shape != (T, slots)) \
+            or (ids is None and down.shape[0] != 1) \
+            or (weights is not None and (weights.shape != (T, slots)
+                                         or weights.dtype != torch.float32)):
+        raise KernelUnavailable(f"moe_down: y {tuple(y.shape)} {y.dtype}, down "
+                                f"{tuple(down.shape)} {down.dtype}, out {tuple(out.shape)}")
+    lib = build.load("moe")
+    _check(lib.zf_moe_down(_ptr(y), _ptr(down), _dt(y), _ptr(ids), _ptr(weights), _ptr(out), T,
+                           W, ff, slots, 1 if add else 0, _stream()), "moe_down")
+
+
 # ------------------------------------------------------------------------- sampling
 SAMPLE_MAX_TOP_K = 1024
 SAMPLE_ROW_DTYPE = [("temperature", "<f4"), ("top_p", "<f4"), ("min_p", "<f4"), ("top_k", "<i4"),

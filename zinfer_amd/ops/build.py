@@ -24,7 +24,8 @@ from typing import Dict, Iterable, List, Optional
 from ..errors import KernelUnavailable
 
 CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
-MODULES = ("elementwise", "gemm", "attention", "sampling", "randinit")
+MODULES = ("elementwise", "gemm", "attention", "sampling", "randinit", "norms",
+           "sink_attention", "moe")
 HOST_MODULES = ("cache_core",)
 HEADERS = ("zf_common.h", "zf_no_alloc.h")
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall"]

@@ -9,6 +9,8 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Callable, Dict
 
+from . import (embed_position, kv_rows_write, moe_down, moe_gate_up, moe_route, norm_rows,
+               shared_kv_attention)
 from . import (advance_decode, apply_penalties, argmax, argmax_no_alloc, cast, check_tables,
                decode_attention_fused, embed, gather_rows, gemm, gemm_emit, gemm_given,
                gemm_partials, gemm_sum_norm, gemm_swiglu, mfma_loop, norm_gemm, paged_attention,
@@ -63,6 +65,17 @@ KERNELS: Dict[str, KernelEntry] = {
                                 "own: a step's block tables and slots against the pool"),
     "stream_read": KernelEntry(stream_read, "elementwise",
                                "own: the read stream bandwidths are measured against"),
+    "norm_rows": KernelEntry(norm_rows, "norms", "own: layer norm / RMS norm with a bias, stored "
+                             "or added to the stream"),
+    "embed_position": KernelEntry(embed_position, "norms", "own: embedding plus a learned "
+                                  "position row"),
+    "kv_rows_write": KernelEntry(kv_rows_write, "sink_attention", "own: key rows into pages"),
+    "shared_kv_attention": KernelEntry(shared_kv_attention, "sink_attention",
+                                       "own: attention whose values are its keys, with a "
+                                       "silent soft-max term and an output gate"),
+    "moe_route": KernelEntry(moe_route, "moe", "own: router logits, top-k, soft-max of the chosen"),
+    "moe_gate_up": KernelEntry(moe_gate_up, "moe", "own: the chosen experts' gated activations"),
+    "moe_down": KernelEntry(moe_down, "moe", "own: the chosen experts' outputs, weighted"),
     "mfma_loop": KernelEntry(mfma_loop, "gemm",
                              "own: MFMAs alone, the rate the tiled products are measured against"),
 }

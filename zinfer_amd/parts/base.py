@@ -17,7 +17,8 @@ Roles and what each must provide:
                   k ``[T, nKV, hd]`` in place
 * mixer           ``cache_need()`` -> KVNeed | StateNeed | None;
                   ``forward(h[T, H], residual_f32[T, H], step, cache)`` adds its output to
-                  ``residual`` (in 32-bit); optionally ``step_hints`` (what its kernels want
+                  ``residual`` (in 32-bit); a part that says ``stores_output`` also takes
+                  ``accumulate=False`` and then stores it there instead; optionally ``step_hints`` (what its kernels want
                   to know about a step's shape, packed with the step's metadata),
                   ``graph_table_pages`` and ``accept_cache``
 * feed_forward    ``forward(h[T, H], residual_f32[T, H], step)`` adds its output to ``residual``
@@ -50,8 +51,9 @@ class KVNeed:
     last ``window`` positions are ever read, so earlier pages may be given back.  A key row
     is ``head_dim`` wide; a value row ``value_dim`` (None: as wide as a key), so a mixer whose
     values are narrower or wider than its keys (or that keeps one shared latent row:
-    ``n_kv_heads`` 1) gets pools of its own widths.  ``dtype``: what the pools hold (None:
-    the engine's cache dtype)."""
+    ``n_kv_heads`` 1) gets pools of its own widths; ``value_dim`` 0: the values are the keys,
+    there is no value pool.  ``dtype``: what the pools hold (None: the engine's cache
+    dtype)."""
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
@@ -169,6 +171,12 @@ class Norm(Part):
 
     def residual_sum(self, linear, a: torch.Tensor, out: torch.Tensor, step) -> bool:
         return False
+
+    def forward_add(self, x: torch.Tensor, residual: torch.Tensor) -> None:
+        """residual += norm(x) in 32-bit (a norm behind a sublayer); a norm that has no kernel
+        for it says so."""
+        raise ConfigError(f"{type(self).__name__} cannot stand behind a sublayer: it has no "
+                          "kernel that adds its result to the residual stream")
 
 
 class PositionEncoding(Part):

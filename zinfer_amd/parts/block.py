@@ -4,7 +4,7 @@ from typing import Dict
 
 import torch
 
-from ..config.specs import PreNormBlockSpec
+from ..config.specs import PreNormBlockSpec, SandwichNormBlockSpec
 from .base import Block, TensorDecl, build_part, register_part
 
 
@@ -72,4 +72,70 @@ class PreNormBlock(Block):
         step.norm_after = None
 
 
+class SandwichNormBlock(Block):
+    """x += post1(mixer(norm1(x))); x += post2(ff(norm2(x))): a norm before every sublayer and
+    one behind it, ahead of the residual sum.  A sublayer's output is a float32 branch of its
+    own (a part that says ``stores_output`` stores it there; any other part adds it to a
+    branch that was cleared first); the norm behind it reads the branch and adds its result to
+    the stream in one kernel, in 32-bit.  Without a feed-forward the block is its first line."""
+
+    def __init__(self, spec: SandwichNormBlockSpec, ctx, prefix):
+        super().__init__(spec, ctx, prefix)
+        self.mixer_norm = build_part("norm", spec.mixer_norm, ctx, prefix + spec.mixer_norm_prefix)
+        self.mixer = build_part("mixer", spec.mixer, ctx, prefix + spec.mixer_prefix)
+        self.mixer_post_norm = build_part("norm", spec.mixer_post_norm, ctx,
+                                          prefix + spec.mixer_post_norm_prefix)
+        self.parts = [self.mixer_norm, self.mixer, self.mixer_post_norm]
+        self.feed_forward = self.ff_norm = self.ff_post_norm = None
+        if spec.feed_forward is not None:
+            self.ff_norm = build_part("norm", spec.ff_norm, ctx, prefix + spec.ff_norm_prefix)
+            self.feed_forward = build_part("feed_forward", spec.feed_forward, ctx,
+                                           prefix + spec.ff_prefix)
+            self.ff_post_norm = build_part("norm", spec.ff_post_norm, ctx,
+                                           prefix + spec.ff_post_norm_prefix)
+            self.parts += [self.ff_norm, self.feed_forward, self.ff_post_norm]
+        self.parts = tuple(self.parts)
+        self.entry_norm = None          # nothing a sum into the stream could leave for it
+        self.graph_safe = all(p.graph_safe for p in self.parts)
+        self.kernel_modules = tuple(sorted({m for p in self.parts for m in p.kernel_modules}))
+
+    def declare(self) -> Dict[str, TensorDecl]:
+        d: Dict[str, TensorDecl] = {}
+        for part in self.parts:
+            d.update(part.declare())
+        return d
+
+    def bind(self, tensors) -> None:
+        for part in self.parts:
+            part.bind(tensors)
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def accept_cache(self, cache) -> None:
+        self.mixer.accept_cache(cache)
+
+    def hint_providers(self):
+        return [q for p in self.parts for q in p.hint_providers()]
+
+    def _sublayer(self, norm, part, post, x, step, *cache) -> None:
+        step.norm_ready = step.norm_after = None
+        h = norm.forward(x, step.scratch("normed", x.shape, self.ctx.act_dtype))
+        branch = step.scratch("branch", x.shape, torch.float32)
+        if getattr(part, "stores_output", False):
+            part.forward(h, branch, step, *cache, accumulate=False)
+        else:
+            branch.zero_()
+            part.forward(h, branch, step, *cache)
+        step.norm_ready = None
+        post.forward_add(branch, x)
+
+    def forward(self, x, step, cache) -> None:
+        self._sublayer(self.mixer_norm, self.mixer, self.mixer_post_norm, x, step, cache)
+        if self.feed_forward is not None:
+            self._sublayer(self.ff_norm, self.feed_forward, self.ff_post_norm, x, step)
+        step.norm_after = None
+
+
 register_part("block", PreNormBlockSpec, PreNormBlock)
+register_part("block", SandwichNormBlockSpec, SandwichNormBlock)

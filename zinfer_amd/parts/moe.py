@@ -1,0 +1,101 @@
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+
+from .. import ops
+from ..config.specs import MoeSpec
+from ..errors import ConfigError
+from .base import FeedForward, TensorDecl, register_part
+from .linear import place_gain, place_matrix
+
+
+class MoeFeedForward(FeedForward):
+    """A mixture of gated experts: the router's logits z = W_r h (+ b_r) are formed in 32-bit,
+    the ``top_k`` largest choose a token's experts, the soft-max over the chosen logits alone
+    weighs them; an expert is W_down act(W_gate h, W_up h) with the clamped, gated activation
+    of ``GatedExpertSpec``; an optional shared expert runs for every token and is added with
+    weight 1.  The experts' matrices are stacked at load (gate rows above up rows, expert by
+    expert) so that the kernels find an expert by its number.  Every token's sum runs over its
+    chosen experts in the order the router ranked them, then the shared one."""
+    graph_safe = True
+    stores_output = True
+    kernel_modules = ("moe",)
+
+    def __init__(self, spec: MoeSpec, ctx, prefix):
+        super().__init__(spec, ctx, prefix)
+        if not 1 <= spec.top_k <= spec.n_experts <= ops.MOE_MAX_EXPERTS:
+            raise ConfigError(f"a mixture of {spec.n_experts} experts with {spec.top_k} a token: "
+                              f"1 <= top <= experts <= {ops.MOE_MAX_EXPERTS}")
+
+    def _expert_names(self, prefix: str):
+        s = self.spec
+        return prefix + s.gate_name, prefix + s.up_name, prefix + s.down_name
+
+    def declare(self) -> Dict[str, TensorDecl]:
+        s, p = self.spec, self.prefix
+        d = {p + s.router_name: TensorDecl((s.n_experts, s.hidden_size))}
+        if s.router_bias:
+            d[p + s.router_bias_name] = TensorDecl((s.n_experts,))
+        groups = [(p + s.expert_prefix.format(e), s.expert) for e in range(s.n_experts)]
+        if s.shared is not None:
+            groups.append((p + s.shared_prefix, s.shared))
+        for prefix, ex in groups:
+            g, u, dn = self._expert_names(prefix)
+            d[g] = TensorDecl((ex.intermediate_size, s.hidden_size))
+            d[u] = TensorDecl((ex.intermediate_size, s.hidden_size))
+            d[dn] = TensorDecl((s.hidden_size, ex.intermediate_size))
+        return d
+
+    def _stack(self, tensors, prefixes):
+        """(gate_up [E, 2 ff, W], down [E, W, ff]) of the experts under ``prefixes``, on the
+        device in the compute dtype, built expert by expert."""
+        gate_up, down = [], []
+        for prefix in prefixes:
+            g, u, dn = (tensors[n] for n in self._expert_names(prefix))
+            if g.dtype != u.dtype:
+                g, u = g.float(), u.float()
+            gate_up.append(place_matrix(torch.cat([g, u], dim=0), self.ctx))
+            down.append(place_matrix(dn, self.ctx))
+        dtypes = {t.dtype for t in gate_up + down}
+        if len(dtypes) > 1:
+            gate_up, down = [t.float() for t in gate_up], [t.float() for t in down]
+        return torch.stack(gate_up).contiguous(), torch.stack(down).contiguous()
+
+    def bind(self, tensors) -> None:
+        s, p = self.spec, self.prefix
+        # the router's logits are 32-bit numbers: its matrix is widened once
+        self.router = place_gain(tensors[p + s.router_name], self.ctx)
+        self.router_bias = place_gain(tensors[p + s.router_bias_name], self.ctx) \
+            if s.router_bias else None
+        self.gate_up, self.down = self._stack(
+            tensors, [p + s.expert_prefix.format(e) for e in range(s.n_experts)])
+        if s.shared is not None:
+            self.shared_gate_up, self.shared_down = self._stack(tensors, [p + s.shared_prefix])
+
+    def forward(self, h, residual, step, accumulate: bool = True) -> None:
+        s = self.spec
+        if hasattr(h, "materialize"):
+            h = h.materialize()
+        T = h.shape[0]
+        dtype = self.gate_up.dtype
+        if h.dtype != dtype:
+            raise ConfigError(f"the experts are held in {dtype}, the activations in {h.dtype}")
+        ids = step.scratch("moe_ids", (T, s.top_k), torch.int32)
+        share = step.scratch("moe_share", (T, s.top_k), torch.float32)
+        ops.moe_route(h, self.router, self.router_bias, ids, share)
+        ex = s.expert
+        y = step.scratch("moe_act", (T, s.top_k, ex.intermediate_size), dtype)
+        ops.moe_gate_up(h, self.gate_up, ids, y, float(ex.limit or 0.0), float(ex.alpha),
+                        float(ex.shift))
+        ops.moe_down(y, self.down, ids, share, residual, add=accumulate)
+        if s.shared is not None:
+            sh = s.shared
+            ys = step.scratch("moe_shared_act", (T, 1, sh.intermediate_size), dtype)
+            ops.moe_gate_up(h, self.shared_gate_up, None, ys, float(sh.limit or 0.0),
+                            float(sh.alpha), float(sh.shift))
+            ops.moe_down(ys, self.shared_down, None, None, residual, add=True)
+
+
+register_part("feed_forward", MoeSpec, MoeFeedForward)

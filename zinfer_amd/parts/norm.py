@@ -5,7 +5,7 @@ from typing import Dict
 import torch
 
 from .. import ops
-from ..config.specs import RmsNormSpec
+from ..config.specs import LayerNormSpec, RmsNormSpec
 from .base import Norm, TensorDecl, register_part
 from .linear import place_gain
 
@@ -125,4 +125,36 @@ class LazyRmsNorm:
         return True
 
 
+class LayerNorm(Norm):
+    """n = (x - mean) / sqrt(mean((x - mean)^2) + eps) * w + b, all in 32-bit; reads the float32
+    residual stream (or a branch's float32 output), writes the activation dtype, or adds its
+    result to a float32 destination (``forward_add``: a norm after a sublayer, ahead of the
+    residual sum).  Not centred it is an RMS norm with a bias."""
+    graph_safe = True
+    kernel_modules = ("norms",)
+
+    def declare(self) -> Dict[str, TensorDecl]:
+        s = self.spec
+        d = {self.prefix + s.weight_name: TensorDecl((s.width,), init="gain")}
+        if s.bias_name is not None:
+            d[self.prefix + s.bias_name] = TensorDecl((s.width,))
+        return d
+
+    def bind(self, tensors) -> None:
+        s = self.spec
+        self.gain = place_gain(tensors[self.prefix + s.weight_name], self.ctx)
+        self.bias = place_gain(tensors[self.prefix + s.bias_name], self.ctx) \
+            if s.bias_name is not None else None
+
+    def forward(self, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        ops.norm_rows(x, self.gain, self.bias, float(self.spec.eps), out, bool(self.spec.centred))
+        return out
+
+    def forward_add(self, x: torch.Tensor, residual: torch.Tensor) -> None:
+        """residual += norm(x), in 32-bit."""
+        ops.norm_rows(x, self.gain, self.bias, float(self.spec.eps), residual,
+                      bool(self.spec.centred), add=True)
+
+
 register_part("norm", RmsNormSpec, RmsNorm)
+register_part("norm", LayerNormSpec, LayerNorm)
