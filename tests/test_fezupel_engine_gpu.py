@@ -1,0 +1,214 @@
+"""Fezupel models through the engine against ``plain_fezupel``, in 32-bit and in bfloat16:
+whole prompts; most of a prompt and then its last tokens one by one; portions of changing
+size down to two tokens; token by token from the first token on (long decoding: many times
+the windows); mixed batches of four live requests in a pool so small that pages are used
+again (what was given back is overwritten with NaN first); greedy generation through the
+entry point and the scheduler; the replay program on a model folder."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import fezupel_tiny as fz
+import plain_fezupel as P
+import traces
+from gpu_util import DEV
+
+pytestmark = pytest.mark.gpu
+
+# float32: what is left is the order of sums; bfloat16: activations rounded to 8 bits of
+# mantissa some ten times a layer run, against the same bfloat16-rounded weights.  Under
+# bfloat16 a router whose two best logits lie within that rounding may choose another expert
+# than the plain implementation does, which changes that position by more than any rounding:
+# up to one position in twelve may lie outside the bfloat16 tolerance (none in 32-bit).
+# (the bfloat16 error grows by about 0.003 of the largest logit at the median with every run of
+# a layer, three to four times that at the worst position: the tolerance follows the runs)
+TOL = {"float32": 3e-5, "bfloat16": 4e-2}
+
+
+def _tol(name, dtype):
+    runs = len(fz.config_of(name).layer_order())
+    return TOL[dtype] if dtype == "float32" else 0.015 + 0.0125 * runs
+
+
+OUTSIDE = {"float32": 0.0, "bfloat16": 1.0 / 12}
+LENGTHS = {"A": (1, 5, 23, 60, 150), "B": (2, 9, 47, 130), "C": (3, 17, 64), "D": (4, 33, 100, 260)}
+_ref = {}
+
+
+def _requests(name, twice=False):
+    vocab = fz.CONFIGS[name]["vocab"]
+    req = {f"r{i}": fz.tokens(n, vocab, 100 + i) for i, n in enumerate(LENGTHS[name])}
+    if twice:
+        req.update({f"s{i}": fz.tokens(n, vocab, 200 + i)
+                    for i, n in enumerate(reversed(LENGTHS[name]))})
+    return req
+
+
+def _reference(name, requests):
+    w = None
+    out = {}
+    for rid, toks in requests.items():
+        key = (name, tuple(toks))
+        if key not in _ref:
+            w = w or fz.weights_of(name)
+            _ref[key] = P.forward(fz.CONFIGS[name], w, toks).numpy()
+        out[rid] = _ref[key]
+    return out
+
+
+def _engine(name, dtype, num_pages, poison=True, max_requests=4):
+    from zinfer_amd.engine import Engine
+    from zinfer_amd.models.build import build_model
+    store = torch.float32 if dtype == "float32" else torch.bfloat16
+    model = build_model(fz.config_of(name).model_spec(), fz.weights_of(name, dtype=store), dtype, DEV)
+    return Engine(model, page_size=fz.PAGE_SIZE[name], num_pages=num_pages,
+                  max_requests=max_requests, poison_freed=poison)
+
+
+def _replay(eng, steps):
+    from zinfer_amd.engine import StepEntry
+    outputs = {}
+    for st in steps:
+        for e in st["entries"]:
+            held = eng.length(e["id"]) if eng.has_request(e["id"]) else 0
+            assert e["start"] == held
+        logits = eng.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in st["entries"]],
+                          end=st["end"])
+        if logits.shape[0]:
+            outputs[st["step"]] = logits.cpu().numpy().copy()
+    eng.cache.check()
+    assert not eng.cache.requests
+    return outputs
+
+
+def _compare(steps, outputs, ref, vocab, dtype, name="A"):
+    tolerance = _tol(name, dtype)
+    got = traces.collect(steps, outputs, vocab)
+    assert set(got) == set(ref)
+    errs = []
+    for rid in ref:
+        assert got[rid].shape == ref[rid].shape
+        assert np.isfinite(got[rid]).all(), f"{rid}: logits are not finite"
+        err = np.abs(got[rid].astype(np.float64) - ref[rid]).max(axis=1) / np.abs(ref[rid]).max()
+        bad = np.nonzero(err > tolerance)[0]
+        assert bad.size <= OUTSIDE[dtype] * len(err) + (dtype == "bfloat16"), \
+            (f"request {rid}: {bad.size} of {len(err)} positions wrong, the first {bad[0]} "
+             f"(error {err[bad[0]]:.3g} > {tolerance})")
+        errs.append(err)
+    errs = np.concatenate(errs)
+    assert (errs > tolerance).sum() <= OUTSIDE[dtype] * len(errs)
+    return float(np.median(errs)) if dtype == "bfloat16" else float(errs.max())
+
+
+MODES = {"whole": traces.whole,
+         "prefill_then_single": lambda r: traces.prefill_then_single(r, tail=20),
+         "portions": traces.changing_portions, "token_by_token": traces.token_by_token,
+         "mixed": lambda r: traces.mixed(r, decode_tail=9)}
+
+
+@pytest.mark.parametrize("mode", list(MODES))
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(fz.CONFIGS))
+def test_replay_modes(name, dtype, mode):
+    requests = _requests(name, twice=mode == "mixed")
+    steps = MODES[mode](requests)
+    page = fz.PAGE_SIZE[name]
+    # the pool holds what is live at the fullest step and no more
+    pages = (traces.peak_tokens(steps, page) + page - 1) // page
+    eng = _engine(name, dtype, pages)
+    outputs = _replay(eng, steps)
+    worst = _compare(steps, outputs, _reference(name, requests), fz.CONFIGS[name]["vocab"], dtype, name)
+    if mode == "mixed":
+        assert max(len(st["entries"]) for st in steps) == 4
+        for grp in eng.cache.groups:
+            assert grp.pages.handed_out > grp.pages.num_pages, "no page was used again"
+    print(f"{name} {dtype} {mode}: error {worst:.3g}")
+
+
+@pytest.mark.parametrize("name", ["A", "D"])
+def test_cut_and_batch_leave_the_bits(name):
+    """32-bit: a position's logits are the same bits whole, in portions, token by token and
+    beside other requests."""
+    requests = _requests(name)
+    vocab = fz.CONFIGS[name]["vocab"]
+    rows = []
+    for mode in ("whole", "portions", "token_by_token", "mixed"):
+        steps = MODES[mode](requests)
+        eng = _engine(name, "float32", 64, poison=False)
+        rows.append(traces.collect(steps, _replay(eng, steps), vocab))
+    for other in rows[1:]:
+        for rid in rows[0]:
+            assert np.array_equal(rows[0][rid], other[rid]), rid
+
+
+def test_windowed_pages_go_back_while_a_request_runs():
+    """A request far longer than its windows holds a few pages a layer run, not its length."""
+    name = "A"            # windows of 7 and 5 tokens, pages of 16
+    toks = fz.tokens(150, fz.CONFIGS[name]["vocab"], 7)
+    steps = traces.changing_portions({"r": toks}, sizes=(13, 2, 30, 1, 8))
+    eng = _engine(name, "float32", 4)          # 64 tokens of pool for 150 tokens
+    outputs = _replay(eng, steps)
+    _compare(steps, outputs, _reference(name, {"r": toks}), fz.CONFIGS[name]["vocab"], "float32", name)
+
+
+def _write_folder(name, path, store):
+    from zinfer_amd.weights.safetensors_io import write_safetensors
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(fz.CONFIGS[name], f)
+    write_safetensors(os.path.join(path, "model.safetensors"), fz.weights_of(name, dtype=store))
+    return path
+
+
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_greedy_generation_through_entry_point_and_scheduler(name, tmp_path):
+    """Prompts of unequal length generate together; every request's tokens are the plain
+    implementation's arg-max wherever that one is clear."""
+    from zinfer_amd.entrypoints import LLM, SamplingParams
+    path = _write_folder(name, str(tmp_path / name), torch.float32)
+    vocab = fz.CONFIGS[name]["vocab"]
+    prompts = [fz.tokens(n, vocab, 300 + n) for n in (3, 41, 18, 7, 29)]
+    llm = LLM(path, dtype="float32", device=DEV, page_size=fz.PAGE_SIZE[name], max_tokens=512,
+              max_step_tokens=48, chunk_size=16, max_seqs=4)
+    n_new = 14
+    outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=n_new,
+                                                ignore_eos=True))
+    w = fz.weights_of(name)
+    for prompt, got in zip(prompts, outs):
+        assert len(got) == n_new
+        logits = P.forward(fz.CONFIGS[name], w, list(prompt) + list(got))
+        for i, tok in enumerate(got):
+            row = logits[len(prompt) - 1 + i]
+            top2 = torch.topk(row, 2).values
+            if float(top2[0] - top2[1]) > 1e-3 * float(row.abs().max()):
+                assert int(row.argmax()) == tok, f"token {i} of a prompt of {len(prompt)}"
+
+
+def test_replay_program_on_a_model_folder(tmp_path):
+    """``bin/trace_run`` chooses the model class by config.json and writes the logits of a
+    mixed trace; both dtypes."""
+    name = "A"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    requests = _requests(name)
+    steps = traces.mixed(requests, decode_tail=5)
+    text = "".join(json.dumps({k: v for k, v in st.items()}) + "\n" for st in steps)
+    ref = _reference(name, requests)
+    for dtype in ("float32", "bfloat16"):
+        store = torch.float32 if dtype == "float32" else torch.bfloat16
+        path = _write_folder(name, str(tmp_path / dtype), store)
+        out = str(tmp_path / ("out_" + dtype))
+        r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", path,
+                            "--dtype", dtype, "--out", out, "--max-tokens",
+                            str(traces.peak_tokens(steps, 64))],
+                           input=text, capture_output=True, text=True, timeout=300)
+        assert r.returncode == 0, r.stderr[-2000:]
+        done = [l for l in r.stdout.splitlines() if l.startswith("done ")]
+        assert done == [f"done {st['step']}" for st in steps]
+        outputs = {st["step"]: np.fromfile(os.path.join(out, f"{st['step']}.f32"), dtype="<f4")
+                   for st in steps if any(e["want"] for e in st["entries"])}
+        _compare(steps, outputs, ref, fz.CONFIGS[name]["vocab"], dtype, name)
