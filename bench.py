@@ -542,10 +542,216 @@ def main_decode(args) -> int:
     return 0
 
 
+# --------------------------------------------------------------------------- Fezupel beside Qwen3
+# Layer sizes that resemble served mixture-of-experts models; every shape is run beside the dense
+# Qwen3 decoder of the same width, heads, head size, depth and vocabulary whose feed-forward is
+# as wide as the experts one token uses (top * ff + shared ff): the same matrix work a token.
+FEZUPEL_SHAPES = {
+    "small": dict(width=2048, heads=16, kv_heads=4, dim=128, window=2048, experts=32, top=4,
+                  ff=768, shared_ff=1024, layers=4, vocab=32768),
+    "medium": dict(width=4096, heads=32, kv_heads=8, dim=128, window=2048, experts=64, top=8,
+                   ff=1024, shared_ff=2048, layers=4, vocab=32768),
+    "narrow-heads": dict(width=3072, heads=32, kv_heads=8, dim=96, window=1024, experts=16,
+                         top=2, ff=2048, shared_ff=2048, layers=4, vocab=32768),
+}
+
+
+def fezupel_config(sh: dict, max_positions: int) -> dict:
+    layer = {"type": "attention",
+             "mixer": {"heads": sh["heads"], "kv_heads": sh["kv_heads"], "dim": sh["dim"],
+                       "vdim": sh["dim"], "scale": sh["dim"] ** -0.5,
+                       "mask": {"size": sh["window"]}},
+             "mlp": {"kind": "moe", "router": {"experts": sh["experts"], "top": sh["top"]},
+                     "expert": {"ff": sh["ff"], "limit": 7.0},
+                     "shared": {"ff": sh["shared_ff"], "limit": 7.0}}}
+    return {"architecture": "Fezupel", "vocab": sh["vocab"], "width": sh["width"],
+            "max_positions": max_positions, "norm": {"eps": 1e-6},
+            "layers": [layer] * sh["layers"]}
+
+
+def dense_twin(sh: dict, max_positions: int) -> dict:
+    return dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3",
+                num_hidden_layers=sh["layers"], hidden_size=sh["width"],
+                num_attention_heads=sh["heads"], num_key_value_heads=sh["kv_heads"],
+                head_dim=sh["dim"], intermediate_size=sh["top"] * sh["ff"] + sh["shared_ff"],
+                vocab_size=sh["vocab"], rope_theta=1000000.0, rms_norm_eps=1e-6,
+                tie_word_embeddings=False, max_position_embeddings=max_positions,
+                torch_dtype="bfloat16")
+
+
+def _timed(fn, repeats: int = 20) -> float:
+    """Seconds of one call of ``fn`` (launches on the current stream), the mean of ``repeats``
+    between two events after two calls that warm up."""
+    import torch
+    fn()
+    fn()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(repeats):
+        fn()
+    b.record()
+    b.synchronize()
+    return a.elapsed_time(b) * 1e-3 / repeats
+
+
+def fezupel_kernels(sh: dict, T: int, ctx: int, mfma_rate: float, read_bw: float) -> dict:
+    """The new design's kernels alone beside the like kernels of the dense decoder, at ``T``
+    tokens of one sequence that holds ``ctx`` tokens (T = ctx: a prompt; T = 1 x 8 sequences: a
+    decode step), each with the fraction of its bound it reaches: matrix work against the MFMA
+    loop's rate (prompt) or bytes read against the measured read stream (decode)."""
+    import torch
+    import zinfer_amd.ops as ops
+    dev = "cuda:0"
+    W, nH, nKV, hd = sh["width"], sh["heads"], sh["kv_heads"], sh["dim"]
+    E, top, ff, sff = sh["experts"], sh["top"], sh["ff"], sh["shared_ff"]
+    bf = torch.bfloat16
+    decode = T == 1
+    n_seqs = 8 if decode else 1
+    rows = n_seqs * T
+    g = torch.Generator(device=dev).manual_seed(1)
+    rnd = lambda *shape: (torch.randn(shape, generator=g, device=dev) * 0.05).to(bf)
+    i32 = lambda a: torch.tensor(a, dtype=torch.int32, device=dev)
+    pages = (ctx + PAGE - 1) // PAGE
+    table = torch.arange(n_seqs * pages, dtype=torch.int32, device=dev).view(n_seqs, pages)
+    q_start = i32([i * T for i in range(n_seqs + 1)])
+    ctx_len = i32([ctx] * n_seqs)
+    seq_index = i32([i for i in range(n_seqs) for _ in range(T)])
+    out = {}
+    # ---- attention: keys (and values) of ctx tokens per sequence
+    q = rnd(rows, nH * hd)
+    gate = rnd(rows, nH * hd)
+    k_pool = rnd(n_seqs * pages, nKV * PAGE * hd)
+    v_pool = rnd(n_seqs * pages, nKV * PAGE * hd)
+    o = torch.empty((rows, nH * hd), dtype=bf, device=dev)
+    window = sh["window"]
+    seen = min(ctx, window)
+    pairs = n_seqs * (seen if decode else sum(min(i + 1, window) for i in range(T)))
+    att_flops = 4.0 * pairs * hd * nH
+    t_new = _timed(lambda: ops.shared_kv_attention(q, gate, k_pool, table, q_start, ctx_len,
+                                                   seq_index, o, hd ** -0.5, window, True, nH,
+                                                   nKV, hd, PAGE, ctx))
+    t_old = _timed(lambda: ops.paged_attention(q, k_pool, v_pool, table, q_start, ctx_len,
+                                               seq_index, o, hd ** -0.5, window, nH, nKV, hd,
+                                               PAGE, T, ctx))
+    if decode:
+        kb = n_seqs * seen * nKV * hd * 2
+        out["attention"] = {"fezupel_us": round(t_new * 1e6, 1), "qwen3_us": round(t_old * 1e6, 1),
+                            "fezupel_frac_of_read": round(kb / t_new / read_bw, 4),
+                            "qwen3_frac_of_read": round(2 * kb / t_old / read_bw, 4)}
+    else:
+        out["attention"] = {"fezupel_us": round(t_new * 1e6, 1), "qwen3_us": round(t_old * 1e6, 1),
+                            "fezupel_frac_of_mfma": round(att_flops / t_new / mfma_rate, 4),
+                            "qwen3_frac_of_mfma": round(att_flops / t_old / mfma_rate, 4)}
+    # ---- feed-forward: the routed experts beside a dense feed-forward of top * ff
+    h = rnd(rows, W)
+    router = torch.randn((E, W), generator=g, device=dev) * 0.05
+    ids = torch.empty((rows, top), dtype=torch.int32, device=dev)
+    share = torch.empty((rows, top), dtype=torch.float32, device=dev)
+    gate_up = rnd(E, 2 * ff, W)
+    down = rnd(E, W, ff)
+    res = torch.zeros((rows, W), dtype=torch.float32, device=dev)
+    moe = _moe_launcher(ops, h, router, ids, share, gate_up, down, res, top, ff)
+    t_moe = _timed(moe)
+    inter = top * ff
+    wgu = ops.pretile_weight(ops.interleave_gate_up(rnd(inter, W), rnd(inter, W)))
+    wd = ops.pretile_weight(rnd(W, inter))
+    act = torch.empty((rows, inter), dtype=bf, device=dev)
+
+    def dense():
+        ops.gemm_swiglu(h, wgu, act, w_tiled=True)
+        ops.gemm(act, wd, res, accumulate=True, w_tiled=True)
+    t_dense = _timed(dense)
+    ff_flops = 2.0 * rows * 3 * inter * W
+    if decode:
+        used = min(E, rows * top)        # at most this many experts' matrices are read
+        mb, db = used * 3 * ff * W * 2, 3 * inter * W * 2
+        out["feed_forward"] = {"fezupel_us": round(t_moe * 1e6, 1), "qwen3_us": round(t_dense * 1e6, 1),
+                               "fezupel_frac_of_read": round(mb / t_moe / read_bw, 4),
+                               "qwen3_frac_of_read": round(db / t_dense / read_bw, 4)}
+    else:
+        out["feed_forward"] = {"fezupel_us": round(t_moe * 1e6, 1), "qwen3_us": round(t_dense * 1e6, 1),
+                               "fezupel_frac_of_mfma": round(ff_flops / t_moe / mfma_rate, 4),
+                               "qwen3_frac_of_mfma": round(ff_flops / t_dense / mfma_rate, 4)}
+    # ---- norms: a layer norm that adds into the stream beside an RMS norm that stores
+    x = torch.randn((rows, W), generator=g, device=dev)
+    gain = torch.ones((W,), device=dev)
+    bias = torch.zeros((W,), device=dev)
+    normed = torch.empty((rows, W), dtype=bf, device=dev)
+    t_ln = _timed(lambda: ops.norm_rows(x, gain, bias, 1e-6, normed, True))
+    t_rms = _timed(lambda: ops.rmsnorm(x, gain, 1e-6, normed))
+    out["norm"] = {"fezupel_us": round(t_ln * 1e6, 1), "qwen3_us": round(t_rms * 1e6, 1)}
+    return out
+
+
+def _moe_launcher(ops, h, router, ids, share, gate_up, down, res, top, ff):
+    import torch
+    rows = h.shape[0]
+    y = torch.empty((rows, top, ff), dtype=h.dtype, device=h.device)
+
+    def run():
+        ops.moe_route(h, router, None, ids, share)
+        ops.moe_experts(h, gate_up, down, ids, share, y, res, 7.0, 1.702, 1.0, add=False)
+    return run
+
+
+def main_fezupel(args) -> int:
+    """Prefill and decode throughput of Fezupel shapes beside the dense Qwen3 decoder of equal
+    size, and the new kernels alone beside the like kernels of that decoder."""
+    import torch
+    import zinfer_amd.ops as ops
+    from zinfer_amd.config import entry_for
+    T, batch, prompt = args.prefill_tokens, args.batch, args.prompt_len
+    max_positions = max(T, prompt + args.steps + args.warmup + 64) + 64
+    read_bw = ops.measure_read_bandwidth("cuda:0")
+    mfma_rate = ops.measure_mfma_rate("cuda:0")
+    names = [args.fezupel_shape] if args.fezupel_shape else list(FEZUPEL_SHAPES)
+    shapes = {}
+    for name in names:
+        sh = FEZUPEL_SHAPES[name]
+        row = {"sizes": sh}
+        for label, raw in (("fezupel", fezupel_config(sh, max_positions)),
+                           ("qwen3", dense_twin(sh, max_positions))):
+            cfg = entry_for(raw).config_type.from_dict(raw)
+            pool = batch * (prompt + args.steps + args.warmup + 64) + T + 256
+            llm = build_llm(raw, args.dtype, args.seed, pool, max(batch, 8),
+                            max_step_tokens=max(T, 2048), multi_step=args.multi_step)
+            t_pre = run_prefill(llm, cfg, T, args.seed + 1)
+            dt, mean_ctx = run_decode(llm, cfg, batch, prompt, args.steps, args.warmup, args.seed + 2)
+            row[label] = {"prefill_tokens_per_s": round(T / t_pre, 1), "prefill_ms": round(t_pre * 1e3, 3),
+                          "decode_tokens_per_s": round(batch * args.steps / dt, 1),
+                          "decode_ms_per_step": round(dt / args.steps * 1e3, 4),
+                          "decode_mean_context": round(mean_ctx, 1)}
+            drop(llm)
+        row["prefill_vs_qwen3"] = round(row["fezupel"]["prefill_tokens_per_s"]
+                                        / row["qwen3"]["prefill_tokens_per_s"], 3)
+        row["decode_vs_qwen3"] = round(row["fezupel"]["decode_tokens_per_s"]
+                                       / row["qwen3"]["decode_tokens_per_s"], 3)
+        if args.dtype == "bfloat16":
+            row["kernels_prefill"] = fezupel_kernels(sh, T, T, mfma_rate, read_bw)
+            row["kernels_decode"] = fezupel_kernels(sh, 1, prompt, mfma_rate, read_bw)
+        ops._workspaces.clear()
+        torch.cuda.empty_cache()
+        shapes[name] = row
+    first = shapes[names[0]]
+    print(json.dumps({
+        "metric": "fezupel_decode_tokens_per_s", "value": first["fezupel"]["decode_tokens_per_s"],
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": first["fezupel"]["decode_ms_per_step"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic", "config": {"model": f"Fezupel {names[0]} shape beside the dense Qwen3 "
+                                                 "decoder of equal size, random weights",
+                                        "batch": batch, "prompt_len": prompt, "prefill_tokens": T,
+                                        "parallelism": "single GPU"},
+        "measured_read_gbs": round(read_bw / 1e9, 1), "mfma_loop_tflops": round(mfma_rate / 1e12, 1),
+        "shapes": shapes}))
+    return 0
+
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "long-context"])
+    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "long-context", "fezupel"])
     ap.add_argument("--shape", default=None, choices=sorted(SHAPES),
                     help="layer sizes (default: 8b for decode, 14b for continuous, 32b for "
                          "long-context)")
@@ -579,6 +785,8 @@ def main() -> int:
     ap.add_argument("--batches", default="1,8,64",
                     help="long-context: the batch sizes decoded at (the pool holds the largest)")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--fezupel-shape", default=None, choices=sorted(FEZUPEL_SHAPES),
+                    help="fezupel: only this shape (default: all of them)")
     ap.add_argument("--no-run-graphs", action="store_true",
                     help="decode steps in a row replay one graph per step instead of one for the run")
     args = ap.parse_args()
@@ -587,7 +795,7 @@ def main() -> int:
               "multi-GPU path")
         return 2
     return {"decode": main_decode, "continuous": main_continuous,
-            "long-context": main_long_context}[args.workload](args)
+            "long-context": main_long_context, "fezupel": main_fezupel}[args.workload](args)
 
 
 if __name__ == "__main__":

@@ -127,6 +127,69 @@ def test_experts(T, W, ff, E, top, dt):
     assert float(gates.max()) > limit
 
 
+@pytest.mark.parametrize("T, W, ff, E, top", [(40, 64, 24, 6, 2), (300, 128, 64, 8, 3),
+                                               (17, 72, 136, 1, 1), (150, 320, 96, 40, 4),
+                                               (260, 64, 8, 3, 3)])
+def test_experts_of_many_tokens_sorted_by_expert(T, W, ff, E, top):
+    """bfloat16, more tokens than stream their experts one by one: the tokens sorted by expert
+    through MFMA tiles against the plain expert, and against the streaming kernels."""
+    dt = torch.bfloat16
+    limit, alpha, shift = 0.6, 1.702, 1.0
+    h = _rand((T, W), 14, dtype=dt)
+    w = {}
+    for e in range(E):
+        w[f"e{e}.gate"] = _rand((ff, W), 120 + e, 2 / W ** 0.5, dt)
+        w[f"e{e}.up"] = _rand((ff, W), 220 + e, 2 / W ** 0.5, dt)
+        w[f"e{e}.down"] = _rand((W, ff), 320 + e, 2 / ff ** 0.5, dt)
+    g = torch.Generator().manual_seed(15)
+    # an expert nobody uses where there are experts to spare; a token names an expert once
+    allowed = [e for e in range(E) if e != 1 or E <= top + 1]
+    ids = torch.stack([torch.tensor(allowed)[torch.randperm(len(allowed), generator=g)[:top]]
+                       for _ in range(T)]).to(torch.int32)
+    share = torch.rand((T, top), generator=g)
+    gate_up = torch.stack([torch.cat([w[f"e{e}.gate"], w[f"e{e}.up"]]) for e in range(E)]).to(DEV)
+    down = torch.stack([w[f"e{e}.down"] for e in range(E)]).to(DEV)
+    assert ops.moe_grouped_covers(h.to(DEV), gate_up) and T > ops.MOE_STREAM_MAX_TOKENS
+    base = _rand((T, W), 16)
+    for add in (False, True):
+        y = torch.empty((T, top, ff), dtype=dt, device=DEV)
+        out = base.to(DEV)
+        ops.moe_experts(h.to(DEV), gate_up, down, ids.to(DEV), share.to(DEV), y, out, limit, alpha,
+                        shift, add=add)
+        y2 = torch.empty((T, top, ff), dtype=dt, device=DEV)
+        out2 = base.to(DEV)
+        ops.moe_gate_up(h.to(DEV), gate_up, ids.to(DEV), y2, limit, alpha, shift)
+        ops.moe_down(y2, down, ids.to(DEV), share.to(DEV), out2, add=add)
+        assert rel_err(out, out2) < 2e-2
+        if T <= 150:
+            ref = base.double() if add else torch.zeros((T, W), dtype=torch.float64)
+            for t in range(T):
+                for s_ in range(top):
+                    ref[t] += share[t, s_].double() * P.clamped_expert(
+                        h[t:t + 1], w, f"e{int(ids[t, s_])}.", limit)[0]
+            assert rel_err(out, ref) < 2e-2
+    # a token's result does not depend on the tokens beside it: the first 20 alone, the same bits
+    if T >= 20:
+        y3 = torch.empty((20, top, ff), dtype=dt, device=DEV)
+        out3 = torch.empty((20, W), dtype=torch.float32, device=DEV)
+        ops.moe_experts(h[:20].to(DEV), gate_up, down, ids[:20].contiguous().to(DEV),
+                        share[:20].contiguous().to(DEV), y3, out3, limit, alpha, shift)
+        out4 = torch.empty((T, W), dtype=torch.float32, device=DEV)
+        ops.moe_experts(h.to(DEV), gate_up, down, ids.to(DEV), share.to(DEV), y, out4, limit,
+                        alpha, shift)
+        assert torch.equal(out3, out4[:20])
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_gated_act(dt):
+    gu = _rand((7, 2 * 24), 17, 2.0, dtype=dt)
+    out = torch.empty((7, 24), dtype=dt, device=DEV)
+    ops.gated_act(gu.to(DEV), out, 1.5, 1.702, 1.0)
+    g = gu[:, :24].double().clamp(max=1.5)
+    u = gu[:, 24:].double().clamp(-1.5, 1.5)
+    assert rel_err(out, g * torch.sigmoid(1.702 * g) * (u + 1)) < tol(dt)
+
+
 # ------------------------------------------------------------------------------ attention
 def _paged(k, n_kv, hd, page_size, seed):
     """Keys [n, n_kv * hd] of one sequence put into a pool through shuffled pages; returns the

@@ -154,6 +154,10 @@ class FezupelConfig:
     def to_dict(self) -> dict:
         return copy.deepcopy(self.raw)
 
+    @property
+    def vocab_size(self) -> int:
+        return self.vocab
+
     # ------------------------------------------------------------------ the model's parts
     def layer_order(self) -> Tuple[int, ...]:
         n = len(self.layers)

@@ -1594,6 +1594,91 @@ def moe_down(y: torch.Tensor, down: torch.Tensor, ids: Optional[torch.Tensor],
                            W, ff, slots, 1 if add else 0, _stream()), "moe_down")
 
 
+@_launches("norm_rope_write")
+def gated_act(gate_up: torch.Tensor, out: torch.Tensor, limit: float, alpha: float,
+              shift: float) -> None:
+    """out[t, j] = g * sigmoid(alpha g) * (u + shift) with g = min(gate_up[t, j], limit) and
+    u = clamp(gate_up[t, ff + j], -limit, limit) (no clamp if limit <= 0)."""
+    _need_gpu(gate_up, out)
+    T, ff = out.shape
+    if gate_up.shape != (T, 2 * ff) or gate_up.dtype != out.dtype:
+        raise KernelUnavailable(f"gated_act: gate_up {tuple(gate_up.shape)}, out {tuple(out.shape)}")
+    lib = build.load("moe")
+    _check(lib.zf_gated_act(_ptr(gate_up), _ptr(out), _dt(out), T, ff, ctypes.c_float(limit),
+                            ctypes.c_float(alpha), ctypes.c_float(shift), _stream()), "gated_act")
+
+
+MOE_TILE_ROWS = 128           # MOE_TILE_ROWS in moe.hip
+MOE_STREAM_MAX_TOKENS = 16    # up to here every (token, expert) streams its own matrices
+
+
+def moe_grouped_covers(h: torch.Tensor, gate_up: torch.Tensor) -> bool:
+    """Whether the MFMA kernels over tokens sorted by expert take these operands: bfloat16,
+    both reduction lengths multiples of 8."""
+    return h.dtype == torch.bfloat16 and gate_up.dtype == torch.bfloat16 \
+        and gate_up.shape[2] % 8 == 0 and (gate_up.shape[1] // 2) % 8 == 0
+
+
+def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, ids: torch.Tensor,
+                weights: torch.Tensor, y: torch.Tensor, out: torch.Tensor, limit: float,
+                alpha: float, shift: float, add: bool = False) -> None:
+    """out[t] (=, +=) sum over s of weights[t, s] * expert ids[t, s] applied to h[t]
+    (``moe_gate_up`` then ``moe_down``), with ``y`` [T, top, ff] as work space.  A few tokens
+    stream each chosen expert's matrices (one workgroup row per token and slot); more tokens,
+    in bfloat16, are sorted by expert and run through MFMA tiles of ``MOE_TILE_ROWS`` pairs
+    (``moe_sort``, ``moe_grouped`` twice, ``moe_combine``).  Either way a token's result
+    depends on that token alone."""
+    T, W = h.shape
+    if T > MOE_STREAM_MAX_TOKENS and moe_grouped_covers(h, gate_up):
+        moe_grouped(h, gate_up, down, ids, weights, y, out, limit, alpha, shift, add)
+        return
+    moe_gate_up(h, gate_up, ids, y, limit, alpha, shift)
+    moe_down(y, down, ids, weights, out, add=add)
+
+
+@_launches("products")
+def moe_grouped(h, gate_up, down, ids, weights, y, out, limit, alpha, shift, add=False) -> None:
+    """The many-token form of ``moe_experts`` (bfloat16; see there)."""
+    _need_gpu(h, gate_up, down, ids, weights, y, out)
+    _i32(ids, "ids")
+    T, W = h.shape
+    E, ff2, _ = gate_up.shape
+    ff = ff2 // 2
+    top = ids.shape[1]
+    if not moe_grouped_covers(h, gate_up) or down.dtype != torch.bfloat16 \
+            or gate_up.shape != (E, 2 * ff, W) or down.shape != (E, W, ff) \
+            or ids.shape != (T, top) or weights.shape != (T, top) \
+            or weights.dtype != torch.float32 or y.dtype != torch.bfloat16 \
+            or y.numel() != T * top * ff or not y.is_contiguous() \
+            or out.shape != (T, W) or out.dtype != torch.float32 or not 0 < E <= MOE_MAX_EXPERTS:
+        raise KernelUnavailable(f"moe_grouped: h {tuple(h.shape)} {h.dtype}, gate_up "
+                                f"{tuple(gate_up.shape)}, down {tuple(down.shape)}, ids "
+                                f"{tuple(ids.shape)}, y {tuple(y.shape)} {y.dtype}")
+    P = T * top
+    max_tiles = (P + MOE_TILE_ROWS - 1) // MOE_TILE_ROWS + E
+    # places of the pairs, the tiles' list and the experts' 32-bit outputs, kept across steps
+    table = _workspace("moe_table", 2 * P + 3 * max_tiles + 4, torch.int32, h.device)
+    o = _workspace("moe_out", P * W, torch.float32, h.device)
+    sorted_, place = table[:P], table[P:2 * P]
+    t0 = 2 * P
+    tile_expert, tile_row0 = table[t0:t0 + max_tiles], table[t0 + max_tiles:t0 + 2 * max_tiles]
+    tile_rows = table[t0 + 2 * max_tiles:t0 + 3 * max_tiles]
+    n_tiles = table[t0 + 3 * max_tiles:]
+    lib = build.load("moe")
+    st = _stream()
+    _check(lib.zf_moe_sort(_ptr(ids), P, E, _ptr(sorted_), _ptr(place), _ptr(tile_expert),
+                           _ptr(tile_row0), _ptr(tile_rows), _ptr(n_tiles), st), "moe_sort")
+    lim, al, sh = ctypes.c_float(limit), ctypes.c_float(alpha), ctypes.c_float(shift)
+    _check(lib.zf_moe_grouped(_ptr(h), ctypes.c_longlong(W), _ptr(sorted_), top, _ptr(gate_up),
+                              _ptr(tile_expert), _ptr(tile_row0), _ptr(tile_rows), _ptr(n_tiles),
+                              _ptr(y), max_tiles, ff, W, 1, lim, al, sh, st), "moe_grouped (gate, up)")
+    _check(lib.zf_moe_grouped(_ptr(y), ctypes.c_longlong(ff), _ptr(sorted_), top, _ptr(down),
+                              _ptr(tile_expert), _ptr(tile_row0), _ptr(tile_rows), _ptr(n_tiles),
+                              _ptr(o), max_tiles, W, ff, 0, lim, al, sh, st), "moe_grouped (down)")
+    _check(lib.zf_moe_combine(_ptr(o), _ptr(place), _ptr(weights), _ptr(out), T, W, top,
+                              1 if add else 0, st), "moe_combine")
+
+
 # ------------------------------------------------------------------------- sampling
 SAMPLE_MAX_TOP_K = 1024
 SAMPLE_ROW_DTYPE = [("temperature", "<f4"), ("top_p", "<f4"), ("min_p", "<f4"), ("top_k", "<i4"),

@@ -9,6 +9,7 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Callable, Dict
 
+from . import (gated_act, moe_grouped)
 from . import (embed_position, kv_rows_write, moe_down, moe_gate_up, moe_route, norm_rows,
                shared_kv_attention)
 from . import (advance_decode, apply_penalties, argmax, argmax_no_alloc, cast, check_tables,
@@ -76,6 +77,9 @@ KERNELS: Dict[str, KernelEntry] = {
     "moe_route": KernelEntry(moe_route, "moe", "own: router logits, top-k, soft-max of the chosen"),
     "moe_gate_up": KernelEntry(moe_gate_up, "moe", "own: the chosen experts' gated activations"),
     "moe_down": KernelEntry(moe_down, "moe", "own: the chosen experts' outputs, weighted"),
+    "moe_grouped": KernelEntry(moe_grouped, "moe", "own: the chosen experts over tokens sorted "
+                               "by expert, MFMA tiles"),
+    "gated_act": KernelEntry(gated_act, "moe", "own: the experts' activation alone"),
     "mfma_loop": KernelEntry(mfma_loop, "gemm",
                              "own: MFMAs alone, the rate the tiled products are measured against"),
 }

@@ -8,7 +8,7 @@ from .. import ops
 from ..config.specs import MoeSpec
 from ..errors import ConfigError
 from .base import FeedForward, TensorDecl, register_part
-from .linear import place_gain, place_matrix
+from .linear import Linear, place_gain, place_matrix
 
 
 class MoeFeedForward(FeedForward):
@@ -21,7 +21,7 @@ class MoeFeedForward(FeedForward):
     chosen experts in the order the router ranked them, then the shared one."""
     graph_safe = True
     stores_output = True
-    kernel_modules = ("moe",)
+    kernel_modules = ("gemm", "moe")
 
     def __init__(self, spec: MoeSpec, ctx, prefix):
         super().__init__(spec, ctx, prefix)
@@ -72,7 +72,9 @@ class MoeFeedForward(FeedForward):
         self.gate_up, self.down = self._stack(
             tensors, [p + s.expert_prefix.format(e) for e in range(s.n_experts)])
         if s.shared is not None:
-            self.shared_gate_up, self.shared_down = self._stack(tensors, [p + s.shared_prefix])
+            # the expert every token uses is two plain products around the activation
+            gu, dn = self._stack(tensors, [p + s.shared_prefix])
+            self.shared_gate_up, self.shared_down = Linear(gu[0]), Linear(dn[0])
 
     def forward(self, h, residual, step, accumulate: bool = True) -> None:
         s = self.spec
@@ -87,15 +89,15 @@ class MoeFeedForward(FeedForward):
         ops.moe_route(h, self.router, self.router_bias, ids, share)
         ex = s.expert
         y = step.scratch("moe_act", (T, s.top_k, ex.intermediate_size), dtype)
-        ops.moe_gate_up(h, self.gate_up, ids, y, float(ex.limit or 0.0), float(ex.alpha),
-                        float(ex.shift))
-        ops.moe_down(y, self.down, ids, share, residual, add=accumulate)
+        ops.moe_experts(h, self.gate_up, self.down, ids, share, y, residual,
+                        float(ex.limit or 0.0), float(ex.alpha), float(ex.shift), add=accumulate)
         if s.shared is not None:
             sh = s.shared
-            ys = step.scratch("moe_shared_act", (T, 1, sh.intermediate_size), dtype)
-            ops.moe_gate_up(h, self.shared_gate_up, None, ys, float(sh.limit or 0.0),
-                            float(sh.alpha), float(sh.shift))
-            ops.moe_down(ys, self.shared_down, None, None, residual, add=True)
+            gu = step.scratch("moe_shared_gate_up", (T, 2 * sh.intermediate_size), dtype)
+            self.shared_gate_up.forward(h, gu)
+            ys = step.scratch("moe_shared_act", (T, sh.intermediate_size), dtype)
+            ops.gated_act(gu, ys, float(sh.limit or 0.0), float(sh.alpha), float(sh.shift))
+            self.shared_down.forward(ys, residual, accumulate=True)
 
 
 register_part("feed_forward", MoeSpec, MoeFeedForward)
