@@ -206,15 +206,53 @@ def _paged(k, n_kv, hd, page_size, seed):
     return pool, table, slots
 
 
-def _attend(q, gate, pool, table, n_ctx, n_q, nH, nKV, hd, page_size, scale, window, sink):
+def _attend(q, gate, pool, table, n_ctx, n_q, nH, nKV, hd, page_size, scale, window, sink,
+            mfma=False, n_splits=None):
     """The last ``n_q`` positions of a sequence of ``n_ctx`` keys."""
     dev = lambda a: torch.tensor(a, dtype=torch.int32, device=DEV)
     out = torch.empty((n_q, nH * hd), dtype=q.dtype, device=DEV)
+    if mfma:
+        ops.tied_attention_mfma(q.to(DEV), None if gate is None else gate.to(DEV), pool,
+                                table.view(1, -1).to(DEV), dev([0, n_q]), dev([n_ctx]), out, scale,
+                                window, sink, nH, nKV, hd, page_size, n_q, n_ctx, n_splits=n_splits)
+        return out
     ops.shared_kv_attention(q.to(DEV), None if gate is None else gate.to(DEV), pool,
                             table.view(1, -1).to(DEV), dev([0, n_q]), dev([n_ctx]),
                             dev([0] * n_q), out, scale, window, sink, nH, nKV, hd, page_size,
                             n_ctx)
     return out
+
+
+@pytest.mark.parametrize("nH, nKV, hd, page", [(4, 2, 32, 16), (6, 3, 96, 16), (5, 1, 64, 8),
+                                               (2, 2, 128, 16), (3, 1, 192, 4), (2, 1, 256, 16),
+                                               (40, 2, 32, 16)])
+@pytest.mark.parametrize("window", [0, 1, 5, 32, 33, 100])
+def test_mfma_attention_against_plain(nH, nKV, hd, page, window):
+    """The bfloat16 MFMA kernel: a whole prompt of several tiles, a portion behind a context,
+    single tokens with the context unsplit and split over 2 and 5 workgroups."""
+    dt = torch.bfloat16
+    n = 171
+    q = _rand((n, nH * hd), 130, dtype=dt)
+    k = _rand((n, nKV * hd), 131, dtype=dt)
+    gate = _rand((n, nH * hd), 132, 2.0, dtype=dt)
+    pool, table, _ = _paged(k, nKV, hd, page, 133)
+    scale = 0.7 / hd ** 0.5
+    ref = P.sink_window_attention(q, k, nH, nKV, hd, scale, window if window else 10 ** 6)
+    gated = ref * torch.sigmoid(gate.double())
+    tolerance = 2.0 ** -7
+    out = _attend(q, gate, pool, table, n, n, nH, nKV, hd, page, scale, window, True, mfma=True)
+    assert rel_err(out, gated) < tolerance
+    tail = _attend(q[-50:], gate[-50:], pool, table, n, 50, nH, nKV, hd, page, scale, window, True,
+                   mfma=True)
+    assert rel_err(tail, gated[-50:]) < tolerance
+    for splits in (1, 2, 5):
+        last = _attend(q[-1:], None, pool, table, n, 1, nH, nKV, hd, page, scale, window, True,
+                       mfma=True, n_splits=splits)
+        assert rel_err(last, ref[-1:]) < tolerance
+    nosink = _attend(q[-1:], gate[-1:], pool, table, n, 1, nH, nKV, hd, page, scale, window, False,
+                     mfma=True, n_splits=3)
+    exact = _attend(q[-1:], gate[-1:], pool, table, n, 1, nH, nKV, hd, page, scale, window, False)
+    assert rel_err(nosink, exact.double()) < tolerance
 
 
 @pytest.mark.parametrize("nH, nKV, hd, page", [(4, 2, 12, 16), (6, 3, 96, 16), (20, 1, 10, 4),
@@ -262,28 +300,31 @@ def test_attention_without_the_silent_term_is_a_plain_softmax():
 
 @pytest.mark.parametrize("window, page", [(7, 16), (16, 16), (33, 8), (64, 16), (65, 16)])
 @pytest.mark.parametrize("decode", [False, True])
-def test_a_loud_key_just_inside_and_just_outside_the_window(window, page, decode):
+@pytest.mark.parametrize("mfma", [False, True])
+def test_a_loud_key_just_inside_and_just_outside_the_window(window, page, decode, mfma):
     """Among hundreds of quiet keys one key answers the last query loudly.  Planted at the
     oldest position the window still holds it takes the output; one position earlier it
     must not be seen at all."""
     nH, nKV, hd, n = 2, 1, 32, 300
     for planted, seen in ((n - window, True), (n - window - 1, False)):
-        k = _rand((n, nKV * hd), 37, 0.05)
-        q = _rand((n, nH * hd), 38, 0.05)
-        loud = torch.zeros(hd)
+        dt = torch.bfloat16 if mfma else torch.float32
+        k = _rand((n, nKV * hd), 37, 0.05, dt)
+        q = _rand((n, nH * hd), 38, 0.05, dt)
+        loud = torch.zeros(hd, dtype=dt)
         loud[3] = 6.0
         k[planted] = loud
         q[n - 1] = torch.cat([loud, loud]) * 2.0
         pool, table, _ = _paged(k, nKV, hd, page, 39)
         n_q = 1 if decode else 9
-        out = _attend(q[-n_q:], None, pool, table, n, n_q, nH, nKV, hd, page, 1.0, window, True)
-        got = out[-1].view(nH, hd).cpu()
+        out = _attend(q[-n_q:], None, pool, table, n, n_q, nH, nKV, hd, page, 1.0, window, True,
+                      mfma=mfma)
+        got = out[-1].view(nH, hd).float().cpu()
         if seen:
             assert float(got[0, 3]) > 5.9 and float(got[1, 3]) > 5.9
         else:
             assert float(got.abs().max()) < 0.5
         ref = P.sink_window_attention(q, k, nH, nKV, hd, 1.0, window)[-1]
-        assert rel_err(out[-1], ref) < 2e-5
+        assert rel_err(out[-1], ref) < (2.0 ** -7 if mfma else 2e-5)
 
 
 def test_first_tokens_and_a_far_key_without_a_window():

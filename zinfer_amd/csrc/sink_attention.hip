@@ -177,3 +177,287 @@ extern "C" int zf_shared_kv_attention(const void* q, long long q_stride, const v
                        (bf16_t*)out, scale, window, sink, nH, nKV, hd, page_size, max_pages);
   ZF_CHECK_LAUNCH();
 }
+
+// =====================================================================================
+//  bfloat16 MFMA kernel (head sizes 32, 64, 96, 128, 192, 256; up to 128 query heads per kv
+//  head).  A workgroup takes one kv head and a tile of query positions of one sequence: its
+//  128 rows are (position, head of the group) pairs, 32 to a wave.  Keys come in chunks of 32,
+//  staged once in LDS in two forms, [key][d] and [d][key], and serve both products of all
+//  rows.  As in the other attention kernels the score tile is computed transposed,
+//  S^T = K Q^T (v_mfma_f32_32x32x16_bf16), so that a lane's 16 scores belong to one row and
+//  the soft-max runs in registers in 32-bit; the second product O^T = K^T P^T takes the
+//  weights from those registers as they lie.  Each weight enters it as the sum of two
+//  bfloat16 numbers (its rounding and the rounding of what that leaves), so what the weights
+//  lose against 32 bits is below 2^-16 of each; the running maximum, the sums and the
+//  accumulators are 32-bit.  With n_splits > 1 (few rows, long contexts: decoding) a
+//  workgroup takes one range of the keys and leaves an un-normalised partial result that
+//  tied_attention_merge_kernel combines in split order; the silent term belongs to split 0.
+// =====================================================================================
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 ta_bf16x8_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float ta_f32x16_t;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t ta_u32x4_t;
+
+#define TA_ROWS 128
+#define TA_KEYS 32
+
+template <int HD>
+__global__ __launch_bounds__(256) void tied_attention_mfma_kernel(
+    const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ gate,
+    long long gate_stride, const bf16_t* __restrict__ k_pool, const int* __restrict__ block_table,
+    const int* __restrict__ q_start, const int* __restrict__ ctx_len, bf16_t* __restrict__ out,
+    float* __restrict__ ws_o, float* __restrict__ ws_ml, float scale, int window, int sink,
+    int n_seqs, int nH, int nKV, int page_size, int max_pages, int QT, int n_splits,
+    int split_keys) {
+  constexpr int LDK = HD + 8;              // [key][d]: 16-byte reads of 8 lanes cover all banks
+  constexpr int LDT = TA_KEYS + 4;         // [d][key]
+  constexpr int CH = TA_KEYS * HD / 8;     // 16-byte pieces of a chunk of keys
+  constexpr int PER = (CH + 255) / 256;
+  __shared__ __attribute__((aligned(16))) bf16_t ks[TA_KEYS * LDK];
+  __shared__ __attribute__((aligned(16))) bf16_t kt[HD * LDT];
+
+  // which sequence and which of its tiles of QT positions this workgroup has
+  int s = 0, tile = blockIdx.x;
+  for (; s < n_seqs; ++s) {
+    const int n = (q_start[s + 1] - q_start[s] + QT - 1) / QT;
+    if (tile < n) break;
+    tile -= n;
+  }
+  if (s >= n_seqs) return;
+  const int kvh = blockIdx.y, split = blockIdx.z;
+  const int G = nH / nKV;
+  const int q_len = q_start[s + 1] - q_start[s];
+  const int first = tile * QT;
+  const int npos = min(QT, q_len - first);
+  const int pos0 = ctx_len[s] - q_len + first;
+  const int nrows = npos * G;
+  const int* table = block_table + (size_t)s * max_pages;
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int c = lane % 32, hl = lane / 32;
+
+  // this lane's row: a (position, head) pair; both halves of the wave hold the same rows
+  const int row = wave * 32 + c;
+  const bool row_ok = row < nrows;
+  const int qi = row_ok ? row / G : 0, g = row_ok ? row % G : 0;
+  const int h = kvh * G + g;
+  const int tok = q_start[s] + first + qi;
+  const int pos_r = pos0 + qi;
+  const int lo_r = (window > 0 && pos_r - window + 1 > 0) ? pos_r - window + 1 : 0;
+  const bool wave_on = wave * 32 < nrows;
+
+  ta_bf16x8_t qf[HD / 16];
+  {
+    const bf16_t* qrow = q + (size_t)tok * q_stride + (size_t)h * HD;
+#pragma unroll
+    for (int i = 0; i < HD / 16; ++i) {
+      ta_u32x4_t v = {0u, 0u, 0u, 0u};
+      if (row_ok) v = *(const ta_u32x4_t*)(qrow + 16 * i + 8 * hl);
+      qf[i] = *(const ta_bf16x8_t*)&v;
+    }
+  }
+  ta_f32x16_t acc[HD / 32];
+#pragma unroll
+  for (int i = 0; i < HD / 32; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
+  const bool has_sink = sink && split == 0;
+  float m = has_sink ? 0.f : -INFINITY, l = has_sink ? 1.f : 0.f;
+
+  // the keys any row of the tile sees, from a multiple of 32 on; this split's part of them
+  const int k_first = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+  const int k_last = pos0 + npos - 1;
+  int k_begin = k_first / TA_KEYS * TA_KEYS, k_end = k_last + 1;
+  if (n_splits > 1) {
+    k_begin += split * split_keys;
+    k_end = min(k_end, k_begin + split_keys);
+  }
+
+  ta_u32x4_t stage[PER];
+  auto fetch = [&](int base) {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int ci = tid + i * 256;
+      ta_u32x4_t v = {0u, 0u, 0u, 0u};
+      if (ci < CH) {
+        const int key = base + ci / (HD / 8);
+        if (key <= k_last) {
+          const size_t prow = ((size_t)table[key / page_size] * nKV + kvh) * page_size + key % page_size;
+          v = *(const ta_u32x4_t*)(k_pool + prow * HD + (ci % (HD / 8)) * 8);
+        }
+      }
+      stage[i] = v;
+    }
+  };
+  if (k_begin < k_end) fetch(k_begin);
+  for (int base = k_begin; base < k_end; base += TA_KEYS) {
+    __syncthreads();                               // the chunk before is done with
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int ci = tid + i * 256;
+      if (ci < CH) {
+        const int j = ci / (HD / 8), d0 = (ci % (HD / 8)) * 8;
+        *(ta_u32x4_t*)(ks + j * LDK + d0) = stage[i];
+        const bf16_t* e = (const bf16_t*)&stage[i];
+#pragma unroll
+        for (int x = 0; x < 8; ++x) kt[(d0 + x) * LDT + j] = e[x];
+      }
+    }
+    __syncthreads();
+    if (base + TA_KEYS < k_end) fetch(base + TA_KEYS);   // in flight while the MFMAs run
+    if (!wave_on) continue;
+    // S^T = K Q^T: this lane gets, for its row, the keys base + 8 (r / 4) + 4 hl + r % 4
+    ta_f32x16_t sc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+#pragma unroll
+    for (int i = 0; i < HD / 16; ++i) {
+      const ta_bf16x8_t kf = *(const ta_bf16x8_t*)(ks + c * LDK + 16 * i + 8 * hl);
+      sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[i], sc, 0, 0, 0);
+    }
+    float cmax = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int key = base + 8 * (r / 4) + 4 * hl + r % 4;
+      const bool seen = row_ok && key <= pos_r && key >= lo_r;
+      sc[r] = seen ? sc[r] * scale : -INFINITY;
+      cmax = fmaxf(cmax, sc[r]);
+    }
+    cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));
+    const float m_new = fmaxf(m, cmax);
+    // nothing seen yet (and no silent term): every weight below is exp(-inf) = 0
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float corr = expf(m - m_use);
+    float psum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      sc[r] = expf(sc[r] - m_use);
+      psum += sc[r];
+    }
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * corr + psum;
+    m = m_new;
+#pragma unroll
+    for (int i = 0; i < HD / 32; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][r] *= corr;
+    // O^T += K^T P^T over the chunk's two groups of 16 keys; the registers 8 t .. 8 t + 7 hold
+    // the weights of the keys 16 t + {0..3, 8..11} + 4 hl, and K^T is read in that same order
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      ta_bf16x8_t p_hi, p_lo;
+#pragma unroll
+      for (int x = 0; x < 8; ++x) {
+        const float p = sc[8 * t + x];
+        const __bf16 hi = (__bf16)p;
+        p_hi[x] = hi;
+        p_lo[x] = (__bf16)(p - (float)hi);
+      }
+#pragma unroll
+      for (int i = 0; i < HD / 32; ++i) {
+        const bf16_t* src = kt + (i * 32 + c) * LDT + 16 * t + 4 * hl;
+        uint2 a0 = *(const uint2*)src, a1 = *(const uint2*)(src + 8);
+        ta_u32x4_t av = {a0.x, a0.y, a1.x, a1.y};
+        const ta_bf16x8_t vf = *(const ta_bf16x8_t*)&av;
+        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, p_hi, acc[i], 0, 0, 0);
+        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, p_lo, acc[i], 0, 0, 0);
+      }
+    }
+  }
+  if (!row_ok) return;
+  // acc[i][r] is element d = 32 i + 8 (r / 4) + 4 hl + r % 4 of this lane's row
+  if (n_splits > 1) {
+    const size_t slot = ((size_t)tok * nH + h) * n_splits + split;
+    float* po = ws_o + slot * HD;
+#pragma unroll
+    for (int i = 0; i < HD / 32; ++i)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4)
+        *(float4*)(po + 32 * i + 8 * r4 + 4 * hl) = make_float4(acc[i][4 * r4], acc[i][4 * r4 + 1],
+                                                                acc[i][4 * r4 + 2], acc[i][4 * r4 + 3]);
+    if (hl == 0) {
+      ws_ml[2 * slot] = m;
+      ws_ml[2 * slot + 1] = l;
+    }
+    return;
+  }
+  const float inv = 1.0f / l;
+  bf16_t* orow = out + ((size_t)tok * nH + h) * HD;
+  const bf16_t* grow = gate != nullptr ? gate + (size_t)tok * gate_stride + (size_t)h * HD : nullptr;
+#pragma unroll
+  for (int i = 0; i < HD / 32; ++i)
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4) {
+      const int d = 32 * i + 8 * r4 + 4 * hl;
+      float v[4];
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        v[x] = acc[i][4 * r4 + x] * inv;
+        if (grow != nullptr) v[x] *= 1.0f / (1.0f + expf(-bf16_to_float(grow[d + x])));
+      }
+      *(uint2*)(orow + d) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+    }
+}
+
+// one wave per (token, head): the splits' partials in split order, then the gate
+__global__ __launch_bounds__(ZF_WAVE) void tied_attention_merge_kernel(
+    const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
+    const bf16_t* __restrict__ gate, long long gate_stride, bf16_t* __restrict__ out, int nH,
+    int hd, int n_splits) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const size_t slot0 = ((size_t)t * nH + h) * n_splits;
+  float M = -INFINITY;
+  for (int z = 0; z < n_splits; ++z) M = fmaxf(M, ws_ml[2 * (slot0 + z)]);
+  float L = 0.f;
+  for (int z = 0; z < n_splits; ++z) {
+    const float mz = ws_ml[2 * (slot0 + z)];
+    if (mz != -INFINITY) L += ws_ml[2 * (slot0 + z) + 1] * expf(mz - M);
+  }
+  const float inv = 1.0f / L;
+  for (int d = lane; d < hd; d += ZF_WAVE) {
+    float o = 0.f;
+    for (int z = 0; z < n_splits; ++z) {
+      const float mz = ws_ml[2 * (slot0 + z)];
+      if (mz != -INFINITY) o += ws_o[(slot0 + z) * hd + d] * expf(mz - M);
+    }
+    o *= inv;
+    if (gate != nullptr)
+      o *= 1.0f / (1.0f + expf(-bf16_to_float(gate[(size_t)t * gate_stride + (size_t)h * hd + d])));
+    out[((size_t)t * nH + h) * hd + d] = float_to_bf16(o);
+  }
+}
+
+#define TA_LAUNCH(HD)                                                                            \
+  case HD:                                                                                       \
+    hipLaunchKernelGGL(tied_attention_mfma_kernel<HD>, grid, dim3(256), 0, stream,               \
+                       (const bf16_t*)q, q_stride, (const bf16_t*)gate, gate_stride,             \
+                       (const bf16_t*)k_pool, block_table, q_start, ctx_len, (bf16_t*)out, ws_o, \
+                       ws_ml, scale, window, sink, n_seqs, nH, nKV, page_size, max_pages, QT,    \
+                       n_splits, split_keys);                                                    \
+    break;
+
+// n_tiles: an upper bound of the tiles of QT = max(1, 128 / G) positions over all sequences
+// (workgroups beyond the real number leave at once).  n_splits > 1: ws_o [T * nH * n_splits *
+// hd] and ws_ml [T * nH * n_splits * 2] floats; split_keys a multiple of 32.
+extern "C" int zf_tied_attention_mfma(const void* q, long long q_stride, const void* gate,
+                                      long long gate_stride, const void* k_pool,
+                                      const int* block_table, const int* q_start,
+                                      const int* ctx_len, void* out, float* ws_o, float* ws_ml,
+                                      float scale, int window, int sink, int T, int n_seqs,
+                                      int n_tiles, int nH, int nKV, int hd, int page_size,
+                                      int max_pages, int n_splits, int split_keys,
+                                      hipStream_t stream) {
+  if (T <= 0 || n_tiles <= 0) return 0;
+  if (nKV <= 0 || nH % nKV != 0 || nH / nKV > TA_ROWS || page_size <= 0 || n_splits < 1 ||
+      (n_splits > 1 && (split_keys <= 0 || split_keys % TA_KEYS != 0 || !ws_o || !ws_ml)))
+    return -2;
+  const int G = nH / nKV;
+  const int QT = TA_ROWS / G;
+  dim3 grid(n_tiles, nKV, n_splits);
+  switch (hd) {
+    TA_LAUNCH(32) TA_LAUNCH(64) TA_LAUNCH(96) TA_LAUNCH(128) TA_LAUNCH(192) TA_LAUNCH(256)
+    default: return -3;
+  }
+  if (n_splits > 1)
+    hipLaunchKernelGGL(tied_attention_merge_kernel, dim3(T, nH), dim3(ZF_WAVE), 0, stream, ws_o,
+                       ws_ml, (const bf16_t*)gate, gate_stride, (bf16_t*)out, nH, hd, n_splits);
+  ZF_CHECK_LAUNCH();
+}

@@ -1518,6 +1518,89 @@ def shared_kv_attention(q: torch.Tensor, gate: Optional[torch.Tensor], k_pool: t
         page_size, block_table.shape[1], _stream()), "shared_kv_attention")
 
 
+TIED_MFMA_HEAD_DIMS = (32, 64, 96, 128, 192, 256)
+TIED_MFMA_ROWS = 128          # (position, head) pairs a workgroup of the MFMA kernel takes
+TIED_SPLIT_KEYS = 256         # least keys a split of a decode step's context holds
+
+
+def tied_attention_mfma_covers(dtype, n_heads: int, n_kv_heads: int, head_dim: int) -> bool:
+    """Whether the bfloat16 MFMA kernel for attention whose values are its keys takes the
+    shape; otherwise (and in 32-bit) ``shared_kv_attention``'s kernel runs."""
+    return dtype == torch.bfloat16 and head_dim in TIED_MFMA_HEAD_DIMS \
+        and n_heads // n_kv_heads <= TIED_MFMA_ROWS
+
+
+def tied_attention(q, gate, k_pool, block_table, q_start, ctx_len, seq_index, out, scale, window,
+                   sink, n_heads, n_kv_heads, head_dim, page_size, max_q_len, max_ctx_len) -> None:
+    """``shared_kv_attention`` through the fastest kernel that takes the shape: in bfloat16,
+    for the head sizes of ``TIED_MFMA_HEAD_DIMS``, MFMA tiles of 128 (position, head) pairs
+    (``tied_attention_mfma``); else the 32-bit kernel.  Same arguments, same result up to
+    rounding."""
+    if tied_attention_mfma_covers(q.dtype, n_heads, n_kv_heads, head_dim):
+        tied_attention_mfma(q, gate, k_pool, block_table, q_start, ctx_len, out, scale, window,
+                            sink, n_heads, n_kv_heads, head_dim, page_size, max_q_len, max_ctx_len)
+    else:
+        shared_kv_attention(q, gate, k_pool, block_table, q_start, ctx_len, seq_index, out, scale,
+                            window, sink, n_heads, n_kv_heads, head_dim, page_size, max_ctx_len)
+
+
+@_launches("attention")
+def tied_attention_mfma(q, gate, k_pool, block_table, q_start, ctx_len, out, scale, window, sink,
+                        n_heads, n_kv_heads, head_dim, page_size, max_q_len, max_ctx_len,
+                        n_splits: Optional[int] = None) -> None:
+    """The bfloat16 MFMA form of ``shared_kv_attention`` (see there for the arguments).  Scores
+    and the soft-max are 32-bit; a weight enters the second product as the sum of two bfloat16
+    numbers.  A step in which every sequence brings one token splits each context over
+    ``n_splits`` workgroups (None: by the block table's width and the window, never by the
+    contexts themselves, so that a captured step replays for other contexts) and merges
+    their partial results."""
+    for t in (q, gate, k_pool, block_table, q_start, ctx_len, out):
+        if t is not None and not t.is_cuda:
+            raise KernelUnavailable("the HIP kernels run on GPU tensors only")
+    T = q.shape[0]
+    qs = _columns(q, "tied_attention_mfma: q")
+    gs = _columns(gate, "tied_attention_mfma: gate") if gate is not None else 0
+    if not tied_attention_mfma_covers(q.dtype, n_heads, n_kv_heads, head_dim):
+        raise KernelUnavailable(f"tied_attention_mfma: bfloat16, head_dim of "
+                                f"{TIED_MFMA_HEAD_DIMS}, at most {TIED_MFMA_ROWS} heads a kv head")
+    if q.shape[1] != n_heads * head_dim or out.shape != (T, n_heads * head_dim) \
+            or not out.is_contiguous() or out.dtype != q.dtype or k_pool.dtype != q.dtype \
+            or (gate is not None and (gate.shape != q.shape or gate.dtype != q.dtype)) \
+            or qs % 8 != 0 or gs % 8 != 0 or q.data_ptr() % 16 != 0 \
+            or (gate is not None and gate.data_ptr() % 16 != 0):
+        raise KernelUnavailable("tied_attention_mfma: q, gate and out must be [T, nH * hd] of "
+                                "the pool's dtype, rows aligned to 16 bytes")
+    for t, name in ((block_table, "block_table"), (q_start, "q_start"), (ctx_len, "ctx_len")):
+        _i32(t, name)
+    if n_kv_heads <= 0 or n_heads % n_kv_heads != 0:
+        raise KernelUnavailable("tied_attention_mfma: InvalidGrouping")
+    n_seqs = ctx_len.shape[0]
+    max_pages = block_table.shape[1]
+    if max_ctx_len > max_pages * page_size or q_start.shape[0] != n_seqs + 1 \
+            or block_table.shape[0] != n_seqs or not block_table.is_contiguous():
+        raise KernelUnavailable("tied_attention_mfma: block table or per-sequence arrays do not fit")
+    G = n_heads // n_kv_heads
+    QT = max(1, TIED_MFMA_ROWS // G)
+    n_tiles = (T + QT - 1) // QT + n_seqs
+    keys = max_pages * page_size if window <= 0 else min(max_pages * page_size, window)
+    if n_splits is None:
+        n_splits = 1
+        if max_q_len == 1 and n_seqs * n_kv_heads < 256:
+            n_splits = max(1, min(keys // TIED_SPLIT_KEYS, 512 // (n_seqs * n_kv_heads), 64))
+    split_keys = ((keys + 32 + n_splits - 1) // n_splits + 31) // 32 * 32
+    ws_o = ws_ml = None
+    if n_splits > 1:
+        ws_o = _workspace("tied_o", T * n_heads * n_splits * head_dim, torch.float32, q.device)
+        ws_ml = _workspace("tied_ml", T * n_heads * n_splits * 2, torch.float32, q.device)
+    lib = build.load("sink_attention")
+    _check(lib.zf_tied_attention_mfma(
+        _ptr(q), ctypes.c_longlong(qs), _ptr(gate), ctypes.c_longlong(gs), _ptr(k_pool),
+        _ptr(block_table), _ptr(q_start), _ptr(ctx_len), _ptr(out), _ptr(ws_o), _ptr(ws_ml),
+        ctypes.c_float(scale), int(window), 1 if sink else 0, T, n_seqs, n_tiles, n_heads,
+        n_kv_heads, head_dim, page_size, max_pages, n_splits, split_keys, _stream()),
+        "tied_attention_mfma")
+
+
 # ------------------------------------------------------------------------- mixture of experts
 MOE_MAX_EXPERTS = 1024
 

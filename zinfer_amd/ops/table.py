@@ -9,7 +9,7 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Callable, Dict
 
-from . import (gated_act, moe_grouped)
+from . import (gated_act, moe_grouped, tied_attention_mfma)
 from . import (embed_position, kv_rows_write, moe_down, moe_gate_up, moe_route, norm_rows,
                shared_kv_attention)
 from . import (advance_decode, apply_penalties, argmax, argmax_no_alloc, cast, check_tables,
@@ -74,6 +74,8 @@ KERNELS: Dict[str, KernelEntry] = {
     "shared_kv_attention": KernelEntry(shared_kv_attention, "sink_attention",
                                        "own: attention whose values are its keys, with a "
                                        "silent soft-max term and an output gate"),
+    "tied_attention_mfma": KernelEntry(tied_attention_mfma, "sink_attention",
+                                       "own: the same attention in MFMA tiles (bfloat16)"),
     "moe_route": KernelEntry(moe_route, "moe", "own: router logits, top-k, soft-max of the chosen"),
     "moe_gate_up": KernelEntry(moe_gate_up, "moe", "own: the chosen experts' gated activations"),
     "moe_down": KernelEntry(moe_down, "moe", "own: the chosen experts' outputs, weighted"),

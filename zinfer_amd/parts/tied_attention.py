@@ -87,11 +87,11 @@ class TiedKeyValueAttention(Mixer):
             ops.kv_rows_write(k, kv.slot_mapping, cache.k_pool, s.n_kv_heads, s.head_dim,
                               cache.page_size)
         attn = step.scratch("attn", (T, self.q_width), act)
-        ops.shared_kv_attention(q, gate, cache.k_pool, kv.block_table, step.q_start, step.ctx_len,
-                                step.seq_index, attn, float(self.scale),
-                                0 if s.window is None else int(s.window), bool(s.sink),
-                                s.n_heads, s.n_kv_heads, s.head_dim, cache.page_size,
-                                step.max_ctx_len)
+        ops.tied_attention(q, gate, cache.k_pool, kv.block_table, step.q_start, step.ctx_len,
+                           step.seq_index, attn, float(self.scale),
+                           0 if s.window is None else int(s.window), bool(s.sink),
+                           s.n_heads, s.n_kv_heads, s.head_dim, cache.page_size,
+                           step.max_q_len, step.max_ctx_len)
         self.o.forward(attn, residual, accumulate=accumulate, step=step if accumulate else None)
 
 
