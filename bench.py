@@ -627,9 +627,9 @@ def fezupel_kernels(sh: dict, T: int, ctx: int, mfma_rate: float, read_bw: float
     seen = min(ctx, window)
     pairs = n_seqs * (seen if decode else sum(min(i + 1, window) for i in range(T)))
     att_flops = 4.0 * pairs * hd * nH
-    t_new = _timed(lambda: ops.shared_kv_attention(q, gate, k_pool, table, q_start, ctx_len,
-                                                   seq_index, o, hd ** -0.5, window, True, nH,
-                                                   nKV, hd, PAGE, ctx))
+    t_new = _timed(lambda: ops.tied_attention(q, gate, k_pool, table, q_start, ctx_len,
+                                              seq_index, o, hd ** -0.5, window, True, nH,
+                                              nKV, hd, PAGE, T, ctx))
     t_old = _timed(lambda: ops.paged_attention(q, k_pool, v_pool, table, q_start, ctx_len,
                                                seq_index, o, hd ** -0.5, window, nH, nKV, hd,
                                                PAGE, T, ctx))

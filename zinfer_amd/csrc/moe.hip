@@ -12,7 +12,7 @@
 // token by token; every token's result depends on that token alone and its sums run in a
 // fixed order, so a token gives the same bits whatever else is in the batch:
 //
-//  * moe_route         one wave per token
+//  * moe_route         a workgroup per four tokens
 //  * moe_gate_up       grid (token * slot, groups of outputs): y[t, slot, :] of the expert in
 //                      that slot, the token's row staged in LDS as 32-bit numbers
 //  * moe_down          grid (token, groups of outputs): out[t, n] (=, or += into) the weighted
@@ -23,22 +23,79 @@
 
 #define MOE_MAX_EXPERTS 1024
 
+#define MOE_ROUTE_TOKENS 4     // tokens a workgroup routes: one wave each for the choice
+#define MOE_ROUTE_WAVES 16     // waves of the workgroup: the experts' logits are dealt over them
+
+template <typename T> struct Vec4 {};
+template <> struct Vec4<float> {
+  static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
+    const float4 x = *(const float4*)p;
+    v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+  }
+};
+template <> struct Vec4<bf16_t> {
+  static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[4]) {
+    const uint2 x = *(const uint2*)p;
+    v[0] = __uint_as_float(x.x << 16); v[1] = __uint_as_float(x.x & 0xffff0000u);
+    v[2] = __uint_as_float(x.y << 16); v[3] = __uint_as_float(x.y & 0xffff0000u);
+  }
+};
+
+// A workgroup of 16 waves takes four tokens.  Logits: wave w forms those of the experts w,
+// w + 16, ... for all four tokens at once (a piece of the router's row is loaded once and meets
+// the four tokens' pieces; every token's sum runs over its own row in a fixed order).  Choice:
+// wave w then ranks token w's logits.
 template <typename T>
-__global__ __launch_bounds__(ZF_WAVE) void moe_route_kernel(
+__global__ __launch_bounds__(MOE_ROUTE_WAVES * ZF_WAVE) void moe_route_kernel(
     const T* __restrict__ h, const float* __restrict__ router, const float* __restrict__ bias,
-    int* __restrict__ ids, float* __restrict__ weights, int W, int E, int top) {
-  __shared__ float z[MOE_MAX_EXPERTS], share[MOE_MAX_EXPERTS];
-  __shared__ int chosen[MOE_MAX_EXPERTS];
-  const int t = blockIdx.x, lane = threadIdx.x;
-  const T* row = h + (size_t)t * W;
-  for (int e = 0; e < E; ++e) {
+    int* __restrict__ ids, float* __restrict__ weights, int n_tokens, int W, int E, int top) {
+  __shared__ float zs[MOE_ROUTE_TOKENS][MOE_MAX_EXPERTS], shares[MOE_ROUTE_TOKENS][MOE_MAX_EXPERTS];
+  __shared__ int chosens[MOE_ROUTE_TOKENS][MOE_MAX_EXPERTS];
+  const int wave = threadIdx.x / ZF_WAVE, lane = threadIdx.x % ZF_WAVE;
+  const int t0 = blockIdx.x * MOE_ROUTE_TOKENS;
+  const T* rows[MOE_ROUTE_TOKENS];
+#pragma unroll
+  for (int k = 0; k < MOE_ROUTE_TOKENS; ++k) rows[k] = h + (size_t)min(t0 + k, n_tokens - 1) * W;
+  for (int e = wave; e < E; e += MOE_ROUTE_WAVES) {
     const float* r = router + (size_t)e * W;
-    float dot = 0.f;
-    for (int i = lane; i < W; i += ZF_WAVE) dot = fmaf(load_as_float<T>(row + i), r[i], dot);
-    dot = wave_sum(dot);
-    if (lane == 0) z[e] = dot + (bias != nullptr ? bias[e] : 0.f);
+    float dot[MOE_ROUTE_TOKENS];
+#pragma unroll
+    for (int k = 0; k < MOE_ROUTE_TOKENS; ++k) dot[k] = 0.f;
+    if (W % 4 == 0) {
+#pragma unroll 4
+      for (int i = lane * 4; i < W; i += ZF_WAVE * 4) {
+        const float4 rv = *(const float4*)(r + i);
+#pragma unroll
+        for (int k = 0; k < MOE_ROUTE_TOKENS; ++k) {
+          float x[4];
+          Vec4<T>::load(rows[k] + i, x);
+          dot[k] = fmaf(x[0], rv.x, dot[k]);
+          dot[k] = fmaf(x[1], rv.y, dot[k]);
+          dot[k] = fmaf(x[2], rv.z, dot[k]);
+          dot[k] = fmaf(x[3], rv.w, dot[k]);
+        }
+      }
+    } else {
+      for (int i = lane; i < W; i += ZF_WAVE) {
+        const float rv = r[i];
+#pragma unroll
+        for (int k = 0; k < MOE_ROUTE_TOKENS; ++k)
+          dot[k] = fmaf(load_as_float<T>(rows[k] + i), rv, dot[k]);
+      }
+    }
+    const float be = bias != nullptr ? bias[e] : 0.f;
+#pragma unroll
+    for (int k = 0; k < MOE_ROUTE_TOKENS; ++k) {
+      const float z = wave_sum(dot[k]);
+      if (lane == 0) zs[k][e] = z + be;
+    }
   }
   __syncthreads();
+  const int t = t0 + wave;
+  if (wave >= MOE_ROUTE_TOKENS || t >= n_tokens) return;
+  float* z = zs[wave];
+  float* share = shares[wave];
+  int* chosen = chosens[wave];
   // `top` rounds of: the largest remaining logit, the lowest index among equals
   float first = 0.f, sum = 0.f;
   for (int k = 0; k < top; ++k) {
@@ -58,13 +115,13 @@ __global__ __launch_bounds__(ZF_WAVE) void moe_route_kernel(
     if (k == 0) first = best;
     const float e_k = expf(best - first);       // the first chosen logit is the largest
     sum += e_k;
-    __syncthreads();
     if (lane == 0) {
       chosen[k] = arg;
       share[k] = e_k;
       z[arg] = -INFINITY;
     }
-    __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
   }
   for (int k = lane; k < top; k += ZF_WAVE) {
     ids[(size_t)t * top + k] = chosen[k];
@@ -77,12 +134,13 @@ extern "C" int zf_moe_route(const void* h, int dtype, const float* router, const
                             hipStream_t stream) {
   if (T <= 0) return 0;
   if (E <= 0 || E > MOE_MAX_EXPERTS || top <= 0 || top > E) return -2;
+  const dim3 grid((T + MOE_ROUTE_TOKENS - 1) / MOE_ROUTE_TOKENS), block(MOE_ROUTE_WAVES * ZF_WAVE);
   if (dtype == ZF_F32)
-    hipLaunchKernelGGL(moe_route_kernel<float>, dim3(T), dim3(ZF_WAVE), 0, stream,
-                       (const float*)h, router, bias, ids, weights, W, E, top);
+    hipLaunchKernelGGL(moe_route_kernel<float>, grid, block, 0, stream, (const float*)h, router,
+                       bias, ids, weights, T, W, E, top);
   else
-    hipLaunchKernelGGL(moe_route_kernel<bf16_t>, dim3(T), dim3(ZF_WAVE), 0, stream,
-                       (const bf16_t*)h, router, bias, ids, weights, W, E, top);
+    hipLaunchKernelGGL(moe_route_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)h, router,
+                       bias, ids, weights, T, W, E, top);
   ZF_CHECK_LAUNCH();
 }
 
@@ -161,6 +219,50 @@ __global__ __launch_bounds__(MOE_WAVES * ZF_WAVE) void moe_gate_up_kernel(
   __syncthreads();
   const T* we = gate_up + (size_t)e * 2 * ff * W;
   const int j0 = (blockIdx.y * MOE_WAVES + wave) * MOE_GU_PER_WAVE;
+  if (j0 >= ff) return;
+  if constexpr (sizeof(T) == 2) {
+    if (W % 8 == 0) {
+      // the wave's outputs side by side: eight 16-byte loads in flight for every piece of the
+      // token's row (an output beyond the last repeats the last one and is not stored)
+      float dg[MOE_GU_PER_WAVE], du[MOE_GU_PER_WAVE];
+      const T* gr[MOE_GU_PER_WAVE];
+#pragma unroll
+      for (int o = 0; o < MOE_GU_PER_WAVE; ++o) {
+        dg[o] = du[o] = 0.f;
+        gr[o] = we + (size_t)min(j0 + o, ff - 1) * W;
+      }
+#pragma unroll 2
+      for (int i = lane * 8; i < W; i += ZF_WAVE * 8) {
+        uint4 a[MOE_GU_PER_WAVE], b[MOE_GU_PER_WAVE];
+#pragma unroll
+        for (int o = 0; o < MOE_GU_PER_WAVE; ++o) {
+          a[o] = *(const uint4*)(gr[o] + i);
+          b[o] = *(const uint4*)(gr[o] + (size_t)ff * W + i);
+        }
+        const float4 x0 = *(const float4*)(xs + i), x1 = *(const float4*)(xs + i + 4);
+        const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+#pragma unroll
+        for (int o = 0; o < MOE_GU_PER_WAVE; ++o) {
+          const uint32_t p[4] = {a[o].x, a[o].y, a[o].z, a[o].w};
+          const uint32_t q[4] = {b[o].x, b[o].y, b[o].z, b[o].w};
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            dg[o] = fmaf(__uint_as_float(p[c] << 16), x[2 * c], dg[o]);
+            dg[o] = fmaf(__uint_as_float(p[c] & 0xffff0000u), x[2 * c + 1], dg[o]);
+            du[o] = fmaf(__uint_as_float(q[c] << 16), x[2 * c], du[o]);
+            du[o] = fmaf(__uint_as_float(q[c] & 0xffff0000u), x[2 * c + 1], du[o]);
+          }
+        }
+      }
+#pragma unroll
+      for (int o = 0; o < MOE_GU_PER_WAVE; ++o) {
+        const float g = wave_sum(dg[o]), u = wave_sum(du[o]);
+        if (lane == 0 && j0 + o < ff)
+          store_from_float<T>(y + (size_t)ts * ff + j0 + o, gated_unit(g, u, limit, alpha, shift));
+      }
+      return;
+    }
+  }
   for (int j = j0; j < j0 + MOE_GU_PER_WAVE && j < ff; ++j) {
     const float g = wave_sum(row_dot_lds<T>(we + (size_t)j * W, xs, W, lane));
     const float u = wave_sum(row_dot_lds<T>(we + (size_t)(ff + j) * W, xs, W, lane));
@@ -198,6 +300,57 @@ __global__ __launch_bounds__(MOE_WAVES * ZF_WAVE) void moe_down_kernel(
   const int t = blockIdx.x;
   const int wave = threadIdx.x / ZF_WAVE, lane = threadIdx.x % ZF_WAVE;
   const int n0 = (blockIdx.y * MOE_WAVES + wave) * MOE_DOWN_PER_WAVE;
+  if (n0 >= W) return;
+  if constexpr (sizeof(T) == 2) {
+    if (ff % 8 == 0) {
+      // the wave's outputs side by side; a lane adds its pieces over all slots (in slot order)
+      // before the lanes are added up, so there is one sum over the wave per output
+      float tot[MOE_DOWN_PER_WAVE];
+#pragma unroll
+      for (int o = 0; o < MOE_DOWN_PER_WAVE; ++o) tot[o] = 0.f;
+      for (int s = 0; s < slots; ++s) {
+        const int ts = t * slots + s;
+        const int e = ids != nullptr ? ids[ts] : 0;
+        const float c = weights != nullptr ? weights[ts] : 1.0f;
+        const T* yr = y + (size_t)ts * ff;
+        const T* wr[MOE_DOWN_PER_WAVE];
+#pragma unroll
+        for (int o = 0; o < MOE_DOWN_PER_WAVE; ++o)
+          wr[o] = down + ((size_t)e * W + min(n0 + o, W - 1)) * ff;
+        float part[MOE_DOWN_PER_WAVE];
+#pragma unroll
+        for (int o = 0; o < MOE_DOWN_PER_WAVE; ++o) part[o] = 0.f;
+        for (int i = lane * 8; i < ff; i += ZF_WAVE * 8) {
+          uint4 a[MOE_DOWN_PER_WAVE];
+#pragma unroll
+          for (int o = 0; o < MOE_DOWN_PER_WAVE; ++o) a[o] = *(const uint4*)(wr[o] + i);
+          const uint4 b = *(const uint4*)(yr + i);
+          const uint32_t q[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+          for (int o = 0; o < MOE_DOWN_PER_WAVE; ++o) {
+            const uint32_t p[4] = {a[o].x, a[o].y, a[o].z, a[o].w};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              part[o] = fmaf(__uint_as_float(p[k] << 16), __uint_as_float(q[k] << 16), part[o]);
+              part[o] = fmaf(__uint_as_float(p[k] & 0xffff0000u),
+                             __uint_as_float(q[k] & 0xffff0000u), part[o]);
+            }
+          }
+        }
+#pragma unroll
+        for (int o = 0; o < MOE_DOWN_PER_WAVE; ++o) tot[o] = fmaf(c, part[o], tot[o]);
+      }
+#pragma unroll
+      for (int o = 0; o < MOE_DOWN_PER_WAVE; ++o) {
+        const float total = wave_sum(tot[o]);
+        if (lane == 0 && n0 + o < W) {
+          float* dst = out + (size_t)t * W + n0 + o;
+          *dst = add ? *dst + total : total;
+        }
+      }
+      return;
+    }
+  }
   for (int n = n0; n < n0 + MOE_DOWN_PER_WAVE && n < W; ++n) {
     float total = 0.f;
     for (int s = 0; s < slots; ++s) {
@@ -324,10 +477,16 @@ typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t moe_u32x
 #define MOE_LD (MOE_BK + 8)      // row stride in LDS (bfloat16): 16-byte reads of 8 lanes cover all banks
 
 // 4 waves as 2 x 2: a wave takes 64 of the tile's 128 rows and 32 of the 64 columns of each of
-// the two weight tiles (GATED: gate rows and up rows of the same 64 outputs; else two
-// neighbouring groups of 64 outputs).  v_mfma_f32_32x32x16_bf16: a lane holds row (or column)
-// lane % 32 and k 8 (lane / 32) .. + 8 of an operand, and of the result column lane % 32, rows
-// 8 (r / 4) + 4 (lane / 32) + r % 4.
+// the MOE_NB weight tiles (GATED: the gate rows of MOE_NB / 2 groups of 64 outputs, then the up
+// rows of the same outputs; else MOE_NB neighbouring groups of 64 outputs).  Two tiles, three
+// workgroups to a CU, ran faster than four tiles with one or two, and loads issued one step
+// ahead faster than two.  What bounds the loop with a few hundred rows an expert is the
+// experts' matrices coming from memory: the tiles of one expert are dealt to workgroups whose
+// numbers are equal modulo 8, which share an XCD and so its L2.
+// v_mfma_f32_32x32x16_bf16: a lane holds row (or column) lane % 32 and k 8 (lane / 32) .. + 8
+// of an operand, and of the result column lane % 32, rows 8 (r / 4) + 4 (lane / 32) + r % 4.
+#define MOE_NB 2                 // weight tiles of 64 rows a workgroup holds
+#define MOE_HALF (MOE_NB / 2)
 template <bool GATED>
 __global__ __launch_bounds__(256) void moe_grouped_kernel(
     const bf16_t* __restrict__ a, long long lda, const int* __restrict__ sorted, int top,
@@ -336,19 +495,21 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
     const int* __restrict__ n_tiles, void* __restrict__ out, int N, int K, float limit,
     float alpha, float shift) {
   __shared__ __attribute__((aligned(16))) bf16_t as[MOE_TILE_ROWS * MOE_LD];
-  __shared__ __attribute__((aligned(16))) bf16_t bs[2 * 64 * MOE_LD];
-  const int tile = blockIdx.x;
+  __shared__ __attribute__((aligned(16))) bf16_t bs[MOE_NB * 64 * MOE_LD];
+  // gridDim.x is a multiple of 8: workgroup x takes tile (x % 8) * (gridDim.x / 8) + x / 8, so
+  // that neighbouring tiles (the same expert's) run on one XCD at about the same time
+  const int tile = (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;
   if (tile >= n_tiles[0]) return;
   const int e = tile_expert[tile], row0 = tile_row0[tile], nrows = tile_rows[tile];
-  const int c0 = blockIdx.y * (GATED ? 64 : 128);
+  const int c0 = blockIdx.y * 64 * (GATED ? MOE_HALF : MOE_NB);
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int wm = wave / 2, wn = wave % 2;
 
-  // what this thread stages: rows tid / 8 + 32 i (i < 4) of the pairs' tile and of the two
-  // weight tiles, 8 values at k0 + 8 (tid % 8)
+  // what this thread stages: rows tid / 8 + 32 i of the pairs' tile (i < 4) and of the
+  // weight tiles (i < 2 MOE_NB), 8 values at k0 + 8 (tid % 8)
   const int sr = tid / 8, sk = (tid % 8) * 8;
   const bf16_t* ap[4];
-  const bf16_t* bp[4];
+  const bf16_t* bp[2 * MOE_NB];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r = sr + 32 * i;
@@ -357,59 +518,65 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
       const int src = GATED ? sorted[row0 + r] / top : row0 + r;
       ap[i] = a + (size_t)src * lda;
     }
-    const int br = r % 64, bt = r / 64;              // row of weight tile bt
+  }
+#pragma unroll
+  for (int i = 0; i < 2 * MOE_NB; ++i) {
+    const int r = sr + 32 * i;
+    const int br = r % 64, bt = r / 64;              // row br of weight tile bt
     size_t wrow;
     bool ok;
-    if (GATED) {
-      ok = c0 + br < N;
-      wrow = (size_t)e * 2 * N + (size_t)bt * N + c0 + br;
+    if (GATED) {                                     // the first half of the tiles: gate; then up
+      const int j = c0 + (bt % MOE_HALF) * 64 + br;
+      ok = j < N;
+      wrow = (size_t)e * 2 * N + (size_t)(bt / MOE_HALF) * N + j;
     } else {
-      ok = c0 + bt * 64 + br < N;
-      wrow = (size_t)e * N + c0 + bt * 64 + br;
+      const int n = c0 + bt * 64 + br;
+      ok = n < N;
+      wrow = (size_t)e * N + n;
     }
     bp[i] = ok ? w + wrow * K : nullptr;
   }
-  moe_f32x16_t acc[2][2];
+  moe_f32x16_t acc[2][MOE_NB];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < MOE_NB; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   const moe_u32x4_t zero = {0u, 0u, 0u, 0u};
-  moe_u32x4_t ra[4], rb[4];
+  moe_u32x4_t ra[4], rb[2 * MOE_NB];
   auto fetch = [&](int k0) {
     const bool in_k = k0 + sk < K;                   // K is a multiple of 8
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < 4; ++i)
       ra[i] = (ap[i] != nullptr && in_k) ? *(const moe_u32x4_t*)(ap[i] + k0 + sk) : zero;
+#pragma unroll
+    for (int i = 0; i < 2 * MOE_NB; ++i)
       rb[i] = (bp[i] != nullptr && in_k) ? *(const moe_u32x4_t*)(bp[i] + k0 + sk) : zero;
-    }
   };
   fetch(0);
   for (int k0 = 0; k0 < K; k0 += MOE_BK) {
     __syncthreads();                                 // the tiles of the step before are done with
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      *(moe_u32x4_t*)(as + (sr + 32 * i) * MOE_LD + sk) = ra[i];
-      *(moe_u32x4_t*)(bs + (sr + 32 * i) * MOE_LD + sk) = rb[i];
-    }
+    for (int i = 0; i < 4; ++i) *(moe_u32x4_t*)(as + (sr + 32 * i) * MOE_LD + sk) = ra[i];
+#pragma unroll
+    for (int i = 0; i < 2 * MOE_NB; ++i) *(moe_u32x4_t*)(bs + (sr + 32 * i) * MOE_LD + sk) = rb[i];
     __syncthreads();
     if (k0 + MOE_BK < K) fetch(k0 + MOE_BK);         // in flight while the MFMAs run
 #pragma unroll
     for (int ks = 0; ks < MOE_BK; ks += 16) {
-      moe_bf16x8_t af[2], bf[2];
+      moe_bf16x8_t af[2], bf[MOE_NB];
 #pragma unroll
       for (int i = 0; i < 2; ++i)
         af[i] = *(const moe_bf16x8_t*)(as + (wm * 64 + i * 32 + lane % 32) * MOE_LD + ks + 8 * (lane / 32));
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < MOE_NB; ++j)
         bf[j] = *(const moe_bf16x8_t*)(bs + (j * 64 + wn * 32 + lane % 32) * MOE_LD + ks + 8 * (lane / 32));
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < MOE_NB; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
     }
   }
@@ -421,12 +588,14 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
       const int row = wm * 64 + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4;
       if (row >= nrows) continue;
       if (GATED) {
-        if (c0 + col < N)
-          ((bf16_t*)out)[(size_t)(row0 + row) * N + c0 + col] =
-              float_to_bf16(gated_unit(acc[i][0][r], acc[i][1][r], limit, alpha, shift));
+#pragma unroll
+        for (int j = 0; j < MOE_HALF; ++j)
+          if (c0 + j * 64 + col < N)
+            ((bf16_t*)out)[(size_t)(row0 + row) * N + c0 + j * 64 + col] =
+                float_to_bf16(gated_unit(acc[i][j][r], acc[i][MOE_HALF + j][r], limit, alpha, shift));
       } else {
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < MOE_NB; ++j)
           if (c0 + j * 64 + col < N)
             ((float*)out)[(size_t)(row0 + row) * N + c0 + j * 64 + col] = acc[i][j][r];
       }
@@ -442,12 +611,13 @@ extern "C" int zf_moe_grouped(const void* a, long long lda, const int* sorted, i
                               hipStream_t stream) {
   if (max_tiles <= 0) return 0;
   if (N <= 0 || K <= 0 || K % 8 != 0 || top <= 0) return -2;
+  max_tiles = (max_tiles + 7) / 8 * 8;
   if (gated)
-    hipLaunchKernelGGL(moe_grouped_kernel<true>, dim3(max_tiles, (N + 63) / 64), dim3(256), 0,
+    hipLaunchKernelGGL(moe_grouped_kernel<true>, dim3(max_tiles, (N + 64 * MOE_HALF - 1) / (64 * MOE_HALF)), dim3(256), 0,
                        stream, (const bf16_t*)a, lda, sorted, top, (const bf16_t*)w, tile_expert,
                        tile_row0, tile_rows, n_tiles, out, N, K, limit, alpha, shift);
   else
-    hipLaunchKernelGGL(moe_grouped_kernel<false>, dim3(max_tiles, (N + 127) / 128), dim3(256), 0,
+    hipLaunchKernelGGL(moe_grouped_kernel<false>, dim3(max_tiles, (N + 64 * MOE_NB - 1) / (64 * MOE_NB)), dim3(256), 0,
                        stream, (const bf16_t*)a, lda, sorted, top, (const bf16_t*)w, tile_expert,
                        tile_row0, tile_rows, n_tiles, out, N, K, limit, alpha, shift);
   ZF_CHECK_LAUNCH();

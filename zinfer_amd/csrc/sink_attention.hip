@@ -200,6 +200,13 @@ typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t ta_u32x4
 #define TA_ROWS 128
 #define TA_KEYS 32
 
+// where key j of row d lies in the [d][key] tile: the row's eight groups of four keys are
+// permuted by the row's group of eight, so that the lanes that write one key of 16 groups of
+// rows (and those that read four keys of 32 rows) spread over the banks
+// 2^x for x <= 0 as the bare instruction (-inf gives 0)
+__device__ __forceinline__ float ta_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ int ta_swz(int j, int d) { return (((j >> 2) ^ ((d >> 3) & 7)) << 2) | (j & 3); }
+
 template <int HD>
 __global__ __launch_bounds__(256) void tied_attention_mfma_kernel(
     const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ gate,
@@ -259,6 +266,9 @@ __global__ __launch_bounds__(256) void tied_attention_mfma_kernel(
   for (int i = 0; i < HD / 32; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
+  // scores are kept times log2(e), so that every weight is one v_exp_f32; the silent term's
+  // score 0 stays 0
+  const float scale_log2 = scale * 1.4426950408889634f;
   const bool has_sink = sink && split == 0;
   float m = has_sink ? 0.f : -INFINITY, l = has_sink ? 1.f : 0.f;
 
@@ -271,8 +281,10 @@ __global__ __launch_bounds__(256) void tied_attention_mfma_kernel(
     k_end = min(k_end, k_begin + split_keys);
   }
 
-  ta_u32x4_t stage[PER];
-  auto fetch = [&](int base) {
+  // three chunks of keys are on their way from memory at any time: a workgroup is alone on its
+  // CU when a prompt has few tiles, so nothing else hides that latency
+  ta_u32x4_t st0[PER], st1[PER], st2[PER];
+  auto fetch = [&](ta_u32x4_t (&stage)[PER], int base) {
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int ci = tid + i * 256;
@@ -287,8 +299,7 @@ __global__ __launch_bounds__(256) void tied_attention_mfma_kernel(
       stage[i] = v;
     }
   };
-  if (k_begin < k_end) fetch(k_begin);
-  for (int base = k_begin; base < k_end; base += TA_KEYS) {
+  auto chunk = [&](ta_u32x4_t (&stage)[PER], int base) {
     __syncthreads();                               // the chunk before is done with
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
@@ -298,12 +309,12 @@ __global__ __launch_bounds__(256) void tied_attention_mfma_kernel(
         *(ta_u32x4_t*)(ks + j * LDK + d0) = stage[i];
         const bf16_t* e = (const bf16_t*)&stage[i];
 #pragma unroll
-        for (int x = 0; x < 8; ++x) kt[(d0 + x) * LDT + j] = e[x];
+        for (int x = 0; x < 8; ++x) kt[(d0 + x) * LDT + ta_swz(j, d0)] = e[x];
       }
     }
     __syncthreads();
-    if (base + TA_KEYS < k_end) fetch(base + TA_KEYS);   // in flight while the MFMAs run
-    if (!wave_on) continue;
+    if (base + 3 * TA_KEYS < k_end) fetch(stage, base + 3 * TA_KEYS);
+    if (!wave_on) return;
     // S^T = K Q^T: this lane gets, for its row, the keys base + 8 (r / 4) + 4 hl + r % 4
     ta_f32x16_t sc;
 #pragma unroll
@@ -314,31 +325,43 @@ __global__ __launch_bounds__(256) void tied_attention_mfma_kernel(
       sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[i], sc, 0, 0, 0);
     }
     float cmax = -INFINITY;
+    // a chunk that every row of the wave sees whole needs no mask
+    const bool whole = row_ok && base >= lo_r && base + TA_KEYS - 1 <= pos_r;
+    if (__all(whole)) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int key = base + 8 * (r / 4) + 4 * hl + r % 4;
-      const bool seen = row_ok && key <= pos_r && key >= lo_r;
-      sc[r] = seen ? sc[r] * scale : -INFINITY;
-      cmax = fmaxf(cmax, sc[r]);
+      for (int r = 0; r < 16; ++r) {
+        sc[r] *= scale_log2;
+        cmax = fmaxf(cmax, sc[r]);
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = base + 8 * (r / 4) + 4 * hl + r % 4;
+        const bool seen = row_ok && key <= pos_r && key >= lo_r;
+        sc[r] = seen ? sc[r] * scale_log2 : -INFINITY;
+        cmax = fmaxf(cmax, sc[r]);
+      }
     }
     cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));
     const float m_new = fmaxf(m, cmax);
     // nothing seen yet (and no silent term): every weight below is exp(-inf) = 0
     const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float corr = expf(m - m_use);
+    const float corr = ta_exp2(m - m_use);
     float psum = 0.f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      sc[r] = expf(sc[r] - m_use);
+      sc[r] = ta_exp2(sc[r] - m_use);
       psum += sc[r];
     }
     psum += __shfl_xor(psum, 32, 64);
     l = l * corr + psum;
     m = m_new;
+    if (__any(corr != 1.0f)) {                     // (the maximum of some row moved)
 #pragma unroll
-    for (int i = 0; i < HD / 32; ++i)
+      for (int i = 0; i < HD / 32; ++i)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][r] *= corr;
+        for (int r = 0; r < 16; ++r) acc[i][r] *= corr;
+    }
     // O^T += K^T P^T over the chunk's two groups of 16 keys; the registers 8 t .. 8 t + 7 hold
     // the weights of the keys 16 t + {0..3, 8..11} + 4 hl, and K^T is read in that same order
 #pragma unroll
@@ -353,14 +376,23 @@ __global__ __launch_bounds__(256) void tied_attention_mfma_kernel(
       }
 #pragma unroll
       for (int i = 0; i < HD / 32; ++i) {
-        const bf16_t* src = kt + (i * 32 + c) * LDT + 16 * t + 4 * hl;
-        uint2 a0 = *(const uint2*)src, a1 = *(const uint2*)(src + 8);
+        const bf16_t* src = kt + (i * 32 + c) * LDT;
+        const uint2 a0 = *(const uint2*)(src + ta_swz(16 * t + 4 * hl, i * 32 + c));
+        const uint2 a1 = *(const uint2*)(src + ta_swz(16 * t + 8 + 4 * hl, i * 32 + c));
         ta_u32x4_t av = {a0.x, a0.y, a1.x, a1.y};
         const ta_bf16x8_t vf = *(const ta_bf16x8_t*)&av;
         acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, p_hi, acc[i], 0, 0, 0);
         acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, p_lo, acc[i], 0, 0, 0);
       }
     }
+  };
+  if (k_begin < k_end) fetch(st0, k_begin);
+  if (k_begin + TA_KEYS < k_end) fetch(st1, k_begin + TA_KEYS);
+  if (k_begin + 2 * TA_KEYS < k_end) fetch(st2, k_begin + 2 * TA_KEYS);
+  for (int base = k_begin; base < k_end; base += 3 * TA_KEYS) {
+    chunk(st0, base);
+    if (base + TA_KEYS < k_end) chunk(st1, base + TA_KEYS);
+    if (base + 2 * TA_KEYS < k_end) chunk(st2, base + 2 * TA_KEYS);
   }
   if (!row_ok) return;
   // acc[i][r] is element d = 32 i + 8 (r / 4) + 4 hl + r % 4 of this lane's row
@@ -397,7 +429,8 @@ __global__ __launch_bounds__(256) void tied_attention_mfma_kernel(
     }
 }
 
-// one wave per (token, head): the splits' partials in split order, then the gate
+// one wave per (token, head): the splits' partials in split order (their maxima are scores
+// times log2(e)), then the gate
 __global__ __launch_bounds__(ZF_WAVE) void tied_attention_merge_kernel(
     const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
     const bf16_t* __restrict__ gate, long long gate_stride, bf16_t* __restrict__ out, int nH,
@@ -409,14 +442,14 @@ __global__ __launch_bounds__(ZF_WAVE) void tied_attention_merge_kernel(
   float L = 0.f;
   for (int z = 0; z < n_splits; ++z) {
     const float mz = ws_ml[2 * (slot0 + z)];
-    if (mz != -INFINITY) L += ws_ml[2 * (slot0 + z) + 1] * expf(mz - M);
+    if (mz != -INFINITY) L += ws_ml[2 * (slot0 + z) + 1] * exp2f(mz - M);
   }
   const float inv = 1.0f / L;
   for (int d = lane; d < hd; d += ZF_WAVE) {
     float o = 0.f;
     for (int z = 0; z < n_splits; ++z) {
       const float mz = ws_ml[2 * (slot0 + z)];
-      if (mz != -INFINITY) o += ws_o[(slot0 + z) * hd + d] * expf(mz - M);
+      if (mz != -INFINITY) o += ws_o[(slot0 + z) * hd + d] * exp2f(mz - M);
     }
     o *= inv;
     if (gate != nullptr)
