@@ -327,6 +327,23 @@ def test_a_loud_key_just_inside_and_just_outside_the_window(window, page, decode
         assert rel_err(out[-1], ref) < (2.0 ** -7 if mfma else 2e-5)
 
 
+@pytest.mark.parametrize("mfma", [False, True])
+def test_pages_before_the_window_are_not_touched(mfma):
+    """The block-table entries of pages that lie wholly before the window are -1 (the pages
+    have gone back): no kernel may look them up."""
+    dt = torch.bfloat16 if mfma else torch.float32
+    nH, nKV, hd, page, n, window = 4, 2, 32, 4, 200, 21
+    q, k = _rand((n, nH * hd), 70, dtype=dt), _rand((n, nKV * hd), 71, dtype=dt)
+    pool, table, _ = _paged(k, nKV, hd, page, 72)
+    ref = P.sink_window_attention(q, k, nH, nKV, hd, 0.2, window)
+    for n_q in (1, 7):
+        gone = table.clone()
+        gone[:(n - n_q + 1 - window) // page] = -1         # wholly before the first query's window
+        out = _attend(q[-n_q:], None, pool, gone, n, n_q, nH, nKV, hd, page, 0.2, window, True,
+                      mfma=mfma)
+        assert rel_err(out, ref[-n_q:]) < (2.0 ** -7 if mfma else 2e-5)
+
+
 def test_first_tokens_and_a_far_key_without_a_window():
     """Position 0 sees itself and the silent term only; with no window the first key of a long
     context still counts."""

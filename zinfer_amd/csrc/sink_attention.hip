@@ -291,7 +291,9 @@ __global__ __launch_bounds__(256) void tied_attention_mfma_kernel(
       ta_u32x4_t v = {0u, 0u, 0u, 0u};
       if (ci < CH) {
         const int key = base + ci / (HD / 8);
-        if (key <= k_last) {
+        // (a chunk starts at a multiple of 32: the keys of its first chunk that lie before
+        // the window may be on a page that has gone back, whose table entry is no page)
+        if (key >= k_first && key <= k_last) {
           const size_t prow = ((size_t)table[key / page_size] * nKV + kvh) * page_size + key % page_size;
           v = *(const ta_u32x4_t*)(k_pool + prow * HD + (ci % (HD / 8)) * 8);
         }
