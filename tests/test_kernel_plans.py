@@ -145,6 +145,14 @@ TESTED_AGAINST = {
     "stream_read": "test_kernels_gpu.py:test_stream_read_reads_every_byte_once",
     "mfma_loop": "test_kernels_gpu.py:test_mfma_loop_sums_its_products",
     "check_tables": "test_kernels_gpu.py:test_check_tables_reports_and_never_traps",
+    "norm_rows": "plain_fezupel.py:layer_norm",
+    "embed_position": "test_fezupel_kernels_gpu.py:test_embed_position",
+    "kv_rows_write": "test_fezupel_kernels_gpu.py:test_attention_against_plain",
+    "shared_kv_attention": "plain_fezupel.py:sink_window_attention",
+    "tied_attention_mfma": "plain_fezupel.py:sink_window_attention",
+    "moe_route": "plain_fezupel.py:route", "moe_gate_up": "plain_fezupel.py:clamped_expert",
+    "moe_down": "plain_fezupel.py:clamped_expert", "moe_grouped": "plain_fezupel.py:clamped_expert",
+    "gated_act": "test_fezupel_kernels_gpu.py:test_gated_act",
 }
 
 

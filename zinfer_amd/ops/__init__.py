@@ -1521,6 +1521,7 @@ def shared_kv_attention(q: torch.Tensor, gate: Optional[torch.Tensor], k_pool: t
 TIED_MFMA_HEAD_DIMS = (32, 64, 96, 128, 192, 256)
 TIED_MFMA_ROWS = 128          # (position, head) pairs a workgroup of the MFMA kernel takes
 TIED_SPLIT_KEYS = 256         # least keys a split of a decode step's context holds
+TIED_SPLIT_WORKGROUPS = 512   # splits are made until about this many workgroups run
 
 
 def tied_attention_mfma_covers(dtype, n_heads: int, n_kv_heads: int, head_dim: int) -> bool:
@@ -1586,7 +1587,8 @@ def tied_attention_mfma(q, gate, k_pool, block_table, q_start, ctx_len, out, sca
     if n_splits is None:
         n_splits = 1
         if max_q_len == 1 and n_seqs * n_kv_heads < 256:
-            n_splits = max(1, min(keys // TIED_SPLIT_KEYS, 512 // (n_seqs * n_kv_heads), 64))
+            n_splits = max(1, min(keys // TIED_SPLIT_KEYS,
+                                  TIED_SPLIT_WORKGROUPS // (n_seqs * n_kv_heads), 64))
     split_keys = ((keys + 32 + n_splits - 1) // n_splits + 31) // 32 * 32
     ws_o = ws_ml = None
     if n_splits > 1:
