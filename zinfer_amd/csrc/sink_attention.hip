@@ -439,20 +439,25 @@ __global__ __launch_bounds__(ZF_WAVE) void tied_attention_merge_kernel(
     int hd, int n_splits) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const size_t slot0 = ((size_t)t * nH + h) * n_splits;
-  float M = -INFINITY;
-  for (int z = 0; z < n_splits; ++z) M = fmaxf(M, ws_ml[2 * (slot0 + z)]);
-  float L = 0.f;
-  for (int z = 0; z < n_splits; ++z) {
-    const float mz = ws_ml[2 * (slot0 + z)];
-    if (mz != -INFINITY) L += ws_ml[2 * (slot0 + z) + 1] * exp2f(mz - M);
+  // lane z holds split z's maximum and sum (at most 64 splits); a split without keys has the
+  // maximum -inf and counts for nothing
+  float mz = -INFINITY, lz = 0.f;
+  if (lane < n_splits) {
+    mz = ws_ml[2 * (slot0 + lane)];
+    lz = ws_ml[2 * (slot0 + lane) + 1];
   }
+  const float M = wave_max(mz);
+  __shared__ float w[ZF_WAVE], lw[ZF_WAVE];
+  w[lane] = mz == -INFINITY ? 0.f : exp2f(mz - M);
+  lw[lane] = lz * w[lane];
+  __syncthreads();
+  // the sums in split order
+  float L = 0.f;
+  for (int z = 0; z < n_splits; ++z) L += lw[z];
   const float inv = 1.0f / L;
   for (int d = lane; d < hd; d += ZF_WAVE) {
     float o = 0.f;
-    for (int z = 0; z < n_splits; ++z) {
-      const float mz = ws_ml[2 * (slot0 + z)];
-      if (mz != -INFINITY) o += ws_o[(slot0 + z) * hd + d] * exp2f(mz - M);
-    }
+    for (int z = 0; z < n_splits; ++z) o += ws_o[(slot0 + z) * hd + d] * w[z];
     o *= inv;
     if (gate != nullptr)
       o *= 1.0f / (1.0f + expf(-bf16_to_float(gate[(size_t)t * gate_stride + (size_t)h * hd + d])));
@@ -482,6 +487,7 @@ extern "C" int zf_tied_attention_mfma(const void* q, long long q_stride, const v
                                       hipStream_t stream) {
   if (T <= 0 || n_tiles <= 0) return 0;
   if (nKV <= 0 || nH % nKV != 0 || nH / nKV > TA_ROWS || page_size <= 0 || n_splits < 1 ||
+      n_splits > ZF_WAVE ||
       (n_splits > 1 && (split_keys <= 0 || split_keys % TA_KEYS != 0 || !ws_o || !ws_ml)))
     return -2;
   const int G = nH / nKV;
