@@ -431,6 +431,166 @@ __global__ __launch_bounds__(256) void tied_attention_mfma_kernel(
     }
 }
 
+// ---------------------------------------------------------------- decode: one token a sequence
+// Grid (sequence, kv head, split); every wave of a workgroup is a split of its own: wave w of
+// workgroup z takes the keys [first + (4 z + w) * wave_keys, + wave_keys) of the context (first:
+// the window's first key, down to a multiple of 32), in chunks of 32.  The token's G rows (its
+// query heads of this kv head) are the first G of the 32 columns.  A lane loads the 8 values of
+// its key that its operand of S^T = K Q^T needs straight from the pool (every value of the
+// chunk exactly once in the wave), and writes them transposed into the wave's own LDS tile
+// for O^T = K^T P^T: no barrier between waves anywhere.  Each wave leaves an un-normalised
+// partial (maximum, sum, O) for tied_attention_merge_kernel; the silent term belongs to the
+// first wave of the first workgroup.
+template <int HD>
+__global__ __launch_bounds__(256) void tied_attention_decode_kernel(
+    const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ k_pool,
+    const int* __restrict__ block_table, const int* __restrict__ ctx_len,
+    float* __restrict__ ws_o, float* __restrict__ ws_ml, float scale, int window, int sink,
+    int nH, int nKV, int page_size, int max_pages, int wave_keys) {
+  constexpr int LDT = TA_KEYS + 4;
+  __shared__ __attribute__((aligned(16))) bf16_t kt_all[4 * HD * LDT];
+  const int s = blockIdx.x, kvh = blockIdx.y;
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int c = lane % 32, hl = lane / 32;
+  bf16_t* kt = kt_all + wave * HD * LDT;
+  const int G = nH / nKV;
+  const int split = blockIdx.z * 4 + wave, n_splits = gridDim.z * 4;
+  const int pos = ctx_len[s] - 1;
+  const int k_first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int* table = block_table + (size_t)s * max_pages;
+  const bool row_ok = c < G;
+  const int h = kvh * G + (row_ok ? c : 0);
+
+  ta_bf16x8_t qf[HD / 16];
+  {
+    const bf16_t* qrow = q + (size_t)s * q_stride + (size_t)h * HD;
+#pragma unroll
+    for (int i = 0; i < HD / 16; ++i) {
+      ta_u32x4_t v = {0u, 0u, 0u, 0u};
+      if (row_ok) v = *(const ta_u32x4_t*)(qrow + 16 * i + 8 * hl);
+      qf[i] = *(const ta_bf16x8_t*)&v;
+    }
+  }
+  ta_f32x16_t acc[HD / 32];
+#pragma unroll
+  for (int i = 0; i < HD / 32; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
+  const float scale_log2 = scale * 1.4426950408889634f;
+  const bool has_sink = sink && split == 0;
+  float m = has_sink ? 0.f : -INFINITY, l = has_sink ? 1.f : 0.f;
+
+  const int k_begin = k_first / TA_KEYS * TA_KEYS + split * wave_keys;
+  const int k_end = min(pos + 1, k_begin + wave_keys);
+
+  // this lane's key of a chunk: key base + c, values 16 i + 8 hl .. + 8 of it for every i
+  ta_u32x4_t kf[HD / 16], kn[HD / 16];
+  auto fetch = [&](ta_u32x4_t (&dst)[HD / 16], int base) {
+    const int key = base + c;
+    const bool ok = key >= k_first && key < k_end;
+    size_t prow = 0;
+    if (ok) prow = ((size_t)table[key / page_size] * nKV + kvh) * page_size + key % page_size;
+#pragma unroll
+    for (int i = 0; i < HD / 16; ++i) {
+      ta_u32x4_t v = {0u, 0u, 0u, 0u};
+      if (ok) v = *(const ta_u32x4_t*)(k_pool + prow * HD + 16 * i + 8 * hl);
+      dst[i] = v;
+    }
+  };
+  if (k_begin < k_end) fetch(kf, k_begin);
+  for (int base = k_begin; base < k_end; base += TA_KEYS) {
+    if (base + TA_KEYS < k_end) fetch(kn, base + TA_KEYS);      // in flight while this chunk runs
+    ta_f32x16_t sc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+#pragma unroll
+    for (int i = 0; i < HD / 16; ++i)
+      sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const ta_bf16x8_t*)&kf[i], qf[i], sc, 0, 0, 0);
+    // the chunk transposed into the wave's tile (the reads of the chunk before are done: they
+    // fed MFMAs whose results were used below)
+#pragma unroll
+    for (int i = 0; i < HD / 16; ++i) {
+      const bf16_t* e = (const bf16_t*)&kf[i];
+#pragma unroll
+      for (int x = 0; x < 8; ++x)
+        kt[(16 * i + 8 * hl + x) * LDT + ta_swz(c, 16 * i + 8 * hl)] = e[x];
+    }
+    float cmax = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int key = base + 8 * (r / 4) + 4 * hl + r % 4;
+      const bool seen = row_ok && key >= k_first && key < k_end;
+      sc[r] = seen ? sc[r] * scale_log2 : -INFINITY;
+      cmax = fmaxf(cmax, sc[r]);
+    }
+    cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));
+    const float m_new = fmaxf(m, cmax);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float corr = ta_exp2(m - m_use);
+    float psum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      sc[r] = ta_exp2(sc[r] - m_use);
+      psum += sc[r];
+    }
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * corr + psum;
+    m = m_new;
+#pragma unroll
+    for (int i = 0; i < HD / 32; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][r] *= corr;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();               // the wave's transposed tile is written
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      ta_bf16x8_t p_hi, p_lo;
+#pragma unroll
+      for (int x = 0; x < 8; ++x) {
+        const float p = sc[8 * t + x];
+        const __bf16 hi = (__bf16)p;
+        p_hi[x] = hi;
+        p_lo[x] = (__bf16)(p - (float)hi);
+      }
+#pragma unroll
+      for (int i = 0; i < HD / 32; ++i) {
+        const bf16_t* src = kt + (i * 32 + c) * LDT;
+        const uint2 a0 = *(const uint2*)(src + ta_swz(16 * t + 4 * hl, i * 32 + c));
+        const uint2 a1 = *(const uint2*)(src + ta_swz(16 * t + 8 + 4 * hl, i * 32 + c));
+        ta_u32x4_t av = {a0.x, a0.y, a1.x, a1.y};
+        const ta_bf16x8_t vf = *(const ta_bf16x8_t*)&av;
+        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, p_hi, acc[i], 0, 0, 0);
+        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, p_lo, acc[i], 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    __builtin_amdgcn_wave_barrier();               // the tile is read before it is written again
+#pragma unroll
+    for (int i = 0; i < HD / 16; ++i) kf[i] = kn[i];
+  }
+  if (!row_ok) return;
+  const size_t slot = ((size_t)s * nH + h) * n_splits + split;
+  float* po = ws_o + slot * HD;
+#pragma unroll
+  for (int i = 0; i < HD / 32; ++i)
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4)
+      *(float4*)(po + 32 * i + 8 * r4 + 4 * hl) = make_float4(acc[i][4 * r4], acc[i][4 * r4 + 1],
+                                                              acc[i][4 * r4 + 2], acc[i][4 * r4 + 3]);
+  if (hl == 0) {
+    ws_ml[2 * slot] = m;
+    ws_ml[2 * slot + 1] = l;
+  }
+}
+
+#define TA_DEC_LAUNCH(HD)                                                                        \
+  case HD:                                                                                       \
+    hipLaunchKernelGGL(tied_attention_decode_kernel<HD>, grid, dim3(256), 0, stream,             \
+                       (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, block_table, ctx_len,  \
+                       ws_o, ws_ml, scale, window, sink, nH, nKV, page_size, max_pages,          \
+                       wave_keys);                                                               \
+    break;
+
 // one wave per (token, head): the splits' partials in split order (their maxima are scores
 // times log2(e)), then the gate
 __global__ __launch_bounds__(ZF_WAVE) void tied_attention_merge_kernel(
@@ -500,5 +660,32 @@ extern "C" int zf_tied_attention_mfma(const void* q, long long q_stride, const v
   if (n_splits > 1)
     hipLaunchKernelGGL(tied_attention_merge_kernel, dim3(T, nH), dim3(ZF_WAVE), 0, stream, ws_o,
                        ws_ml, (const bf16_t*)gate, gate_stride, (bf16_t*)out, nH, hd, n_splits);
+  ZF_CHECK_LAUNCH();
+}
+
+// A step in which every sequence brings one token (token s is sequence s's): n_blocks
+// workgroups a (sequence, kv head), every wave a split of wave_keys keys (a multiple of 32);
+// ws_o [n_seqs * nH * 4 n_blocks * hd], ws_ml [n_seqs * nH * 4 n_blocks * 2] floats;
+// 4 n_blocks <= 64; at most 32 query heads a kv head; head sizes up to 128 (the wave's tile and
+// operands in registers).
+extern "C" int zf_tied_attention_decode(const void* q, long long q_stride, const void* gate,
+                                        long long gate_stride, const void* k_pool,
+                                        const int* block_table, const int* ctx_len, void* out,
+                                        float* ws_o, float* ws_ml, float scale, int window,
+                                        int sink, int n_seqs, int nH, int nKV, int hd,
+                                        int page_size, int max_pages, int n_blocks, int wave_keys,
+                                        hipStream_t stream) {
+  if (n_seqs <= 0) return 0;
+  if (nKV <= 0 || nH % nKV != 0 || nH / nKV > 32 || page_size <= 0 || n_blocks < 1 ||
+      4 * n_blocks > ZF_WAVE || wave_keys <= 0 || wave_keys % TA_KEYS != 0 || !ws_o || !ws_ml)
+    return -2;
+  dim3 grid(n_seqs, nKV, n_blocks);
+  switch (hd) {
+    TA_DEC_LAUNCH(32) TA_DEC_LAUNCH(64) TA_DEC_LAUNCH(96) TA_DEC_LAUNCH(128)
+    default: return -3;
+  }
+  hipLaunchKernelGGL(tied_attention_merge_kernel, dim3(n_seqs, nH), dim3(ZF_WAVE), 0, stream,
+                     ws_o, ws_ml, (const bf16_t*)gate, gate_stride, (bf16_t*)out, nH, hd,
+                     4 * n_blocks);
   ZF_CHECK_LAUNCH();
 }

@@ -1522,6 +1522,7 @@ TIED_MFMA_HEAD_DIMS = (32, 64, 96, 128, 192, 256)
 TIED_MFMA_ROWS = 128          # (position, head) pairs a workgroup of the MFMA kernel takes
 TIED_SPLIT_KEYS = 256         # least keys a split of a decode step's context holds
 TIED_SPLIT_WORKGROUPS = 512   # splits are made until about this many workgroups run
+TIED_DECODE_WORKGROUPS = 1024  # the same for the decode kernel (whose every wave is a split)
 
 
 def tied_attention_mfma_covers(dtype, n_heads: int, n_kv_heads: int, head_dim: int) -> bool:
@@ -1551,10 +1552,11 @@ def tied_attention_mfma(q, gate, k_pool, block_table, q_start, ctx_len, out, sca
                         n_splits: Optional[int] = None) -> None:
     """The bfloat16 MFMA form of ``shared_kv_attention`` (see there for the arguments).  Scores
     and the soft-max are 32-bit; a weight enters the second product as the sum of two bfloat16
-    numbers.  A step in which every sequence brings one token splits each context over
-    ``n_splits`` workgroups (None: by the block table's width and the window, never by the
-    contexts themselves, so that a captured step replays for other contexts) and merges
-    their partial results."""
+    numbers.  A step in which every sequence brings one token runs the decode kernel (head
+    sizes up to 128, at most 32 heads a kv head): each context is split over ``n_splits``
+    workgroups of four waves that are splits of their own (None: by the block table's width and
+    the window, never by the contexts themselves, so that a captured step replays for other
+    contexts), and the partial results are merged."""
     for t in (q, gate, k_pool, block_table, q_start, ctx_len, out):
         if t is not None and not t.is_cuda:
             raise KernelUnavailable("the HIP kernels run on GPU tensors only")
@@ -1581,9 +1583,29 @@ def tied_attention_mfma(q, gate, k_pool, block_table, q_start, ctx_len, out, sca
             or block_table.shape[0] != n_seqs or not block_table.is_contiguous():
         raise KernelUnavailable("tied_attention_mfma: block table or per-sequence arrays do not fit")
     G = n_heads // n_kv_heads
+    lib = build.load("sink_attention")
+    keys = max_pages * page_size if window <= 0 else min(max_pages * page_size, window)
+    if max_q_len == 1 and T == n_seqs and head_dim <= 128 and G <= 32:
+        # a decode step: every wave of a workgroup is a split of its own
+        # (``tied_attention_decode_kernel``); about 1024 workgroups, at least 64 keys a wave
+        span = keys + 31                      # the first chunk starts at a multiple of 32
+        blocks = n_splits if n_splits is not None else \
+            max(1, min(TIED_DECODE_WORKGROUPS // max(1, n_seqs * n_kv_heads),
+                       (span + 255) // 256, 16))
+        if not 1 <= blocks <= 16:
+            raise KernelUnavailable("tied_attention_mfma: 1 to 16 workgroups a context")
+        wave_keys = ((span + 4 * blocks - 1) // (4 * blocks) + 31) // 32 * 32
+        ws_o = _workspace("tied_o", T * n_heads * 4 * blocks * head_dim, torch.float32, q.device)
+        ws_ml = _workspace("tied_ml", T * n_heads * 4 * blocks * 2, torch.float32, q.device)
+        _check(lib.zf_tied_attention_decode(
+            _ptr(q), ctypes.c_longlong(qs), _ptr(gate), ctypes.c_longlong(gs), _ptr(k_pool),
+            _ptr(block_table), _ptr(ctx_len), _ptr(out), _ptr(ws_o), _ptr(ws_ml),
+            ctypes.c_float(scale), int(window), 1 if sink else 0, n_seqs, n_heads, n_kv_heads,
+            head_dim, page_size, max_pages, blocks, wave_keys, _stream()),
+            "tied_attention_mfma (decode)")
+        return
     QT = max(1, TIED_MFMA_ROWS // G)
     n_tiles = (T + QT - 1) // QT + n_seqs
-    keys = max_pages * page_size if window <= 0 else min(max_pages * page_size, window)
     if n_splits is None:
         n_splits = 1
         if max_q_len == 1 and n_seqs * n_kv_heads < 256:
@@ -1594,7 +1616,6 @@ def tied_attention_mfma(q, gate, k_pool, block_table, q_start, ctx_len, out, sca
     if n_splits > 1:
         ws_o = _workspace("tied_o", T * n_heads * n_splits * head_dim, torch.float32, q.device)
         ws_ml = _workspace("tied_ml", T * n_heads * n_splits * 2, torch.float32, q.device)
-    lib = build.load("sink_attention")
     _check(lib.zf_tied_attention_mfma(
         _ptr(q), ctypes.c_longlong(qs), _ptr(gate), ctypes.c_longlong(gs), _ptr(k_pool),
         _ptr(block_table), _ptr(q_start), _ptr(ctx_len), _ptr(out), _ptr(ws_o), _ptr(ws_ml),
