@@ -207,14 +207,15 @@ def _paged(k, n_kv, hd, page_size, seed):
 
 
 def _attend(q, gate, pool, table, n_ctx, n_q, nH, nKV, hd, page_size, scale, window, sink,
-            mfma=False, n_splits=None):
+            mfma=False, n_splits=None, shared_tiles=None):
     """The last ``n_q`` positions of a sequence of ``n_ctx`` keys."""
     dev = lambda a: torch.tensor(a, dtype=torch.int32, device=DEV)
     out = torch.empty((n_q, nH * hd), dtype=q.dtype, device=DEV)
     if mfma:
         ops.tied_attention_mfma(q.to(DEV), None if gate is None else gate.to(DEV), pool,
                                 table.view(1, -1).to(DEV), dev([0, n_q]), dev([n_ctx]), out, scale,
-                                window, sink, nH, nKV, hd, page_size, n_q, n_ctx, n_splits=n_splits)
+                                window, sink, nH, nKV, hd, page_size, n_q, n_ctx, n_splits=n_splits,
+                                shared_tiles=shared_tiles)
         return out
     ops.shared_kv_attention(q.to(DEV), None if gate is None else gate.to(DEV), pool,
                             table.view(1, -1).to(DEV), dev([0, n_q]), dev([n_ctx]),
@@ -240,11 +241,16 @@ def test_mfma_attention_against_plain(nH, nKV, hd, page, window):
     ref = P.sink_window_attention(q, k, nH, nKV, hd, scale, window if window else 10 ** 6)
     gated = ref * torch.sigmoid(gate.double())
     tolerance = 2.0 ** -7
-    out = _attend(q, gate, pool, table, n, n, nH, nKV, hd, page, scale, window, True, mfma=True)
-    assert rel_err(out, gated) < tolerance
-    tail = _attend(q[-50:], gate[-50:], pool, table, n, 50, nH, nKV, hd, page, scale, window, True,
-                   mfma=True)
-    assert rel_err(tail, gated[-50:]) < tolerance
+    for tiles in (None, True):          # waves on their own where the shape allows; shared tiles
+        out = _attend(q, gate, pool, table, n, n, nH, nKV, hd, page, scale, window, True, mfma=True,
+                      shared_tiles=tiles)
+        assert rel_err(out, gated) < tolerance
+        tail = _attend(q[-50:], gate[-50:], pool, table, n, 50, nH, nKV, hd, page, scale, window,
+                       True, mfma=True, shared_tiles=tiles)
+        assert rel_err(tail, gated[-50:]) < tolerance
+        one = _attend(q[-1:], gate[-1:], pool, table, n, 1, nH, nKV, hd, page, scale, window, True,
+                      mfma=True, n_splits=2, shared_tiles=tiles)
+        assert rel_err(one, gated[-1:]) < tolerance
     for splits in (1, 2, 5):
         last = _attend(q[-1:], None, pool, table, n, 1, nH, nKV, hd, page, scale, window, True,
                        mfma=True, n_splits=splits)

@@ -441,29 +441,74 @@ __global__ __launch_bounds__(256) void tied_attention_mfma_kernel(
 // for O^T = K^T P^T: no barrier between waves anywhere.  Each wave leaves an un-normalised
 // partial (maximum, sum, O) for tied_attention_merge_kernel; the silent term belongs to the
 // first wave of the first workgroup.
-template <int HD>
-__global__ __launch_bounds__(256) void tied_attention_decode_kernel(
-    const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ k_pool,
-    const int* __restrict__ block_table, const int* __restrict__ ctx_len,
+template <int HD, bool DECODE>
+__global__ __launch_bounds__(256, 2) void tied_attention_wave_kernel(
+    const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ gate,
+    long long gate_stride, const bf16_t* __restrict__ k_pool, const int* __restrict__ block_table,
+    const int* __restrict__ q_start, const int* __restrict__ ctx_len, bf16_t* __restrict__ out,
     float* __restrict__ ws_o, float* __restrict__ ws_ml, float scale, int window, int sink,
-    int nH, int nKV, int page_size, int max_pages, int wave_keys) {
+    int n_seqs, int nH, int nKV, int page_size, int max_pages, int QT, int wave_keys) {
   constexpr int LDT = TA_KEYS + 4;
   __shared__ __attribute__((aligned(16))) bf16_t kt_all[4 * HD * LDT];
-  const int s = blockIdx.x, kvh = blockIdx.y;
+  const int kvh = blockIdx.y;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int c = lane % 32, hl = lane / 32;
   bf16_t* kt = kt_all + wave * HD * LDT;
   const int G = nH / nKV;
-  const int split = blockIdx.z * 4 + wave, n_splits = gridDim.z * 4;
-  const int pos = ctx_len[s] - 1;
-  const int k_first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+
+  // the wave's 32 rows: (position, head of the group) pairs of one sequence
+  int s, tok, pos_r, lo_r, h, split = 0, n_splits = 1;
+  int k_first, k_end;          // the keys the wave walks: [k_first down to a multiple of 32, k_end)
+  bool row_ok;
+  if constexpr (DECODE) {
+    // one token a sequence; the workgroup's four waves are four splits of its context
+    s = blockIdx.x;
+    split = blockIdx.z * 4 + wave;
+    n_splits = gridDim.z * 4;
+    row_ok = c < G;
+    h = kvh * G + (row_ok ? c : 0);
+    tok = s;
+    pos_r = ctx_len[s] - 1;
+    lo_r = (window > 0 && pos_r - window + 1 > 0) ? pos_r - window + 1 : 0;
+    k_first = lo_r;
+    k_end = pos_r + 1;
+  } else {
+    // a tile of QT positions of a sequence; the four waves take 32 rows each, and with
+    // gridDim.z > 1 the z-th part of their keys (a prompt's last rows see the most keys and
+    // its first the fewest: parts even out what the waves have to do, and let a SIMD hold two)
+    split = blockIdx.z;
+    n_splits = gridDim.z;
+    s = 0;
+    int tile = blockIdx.x;
+    for (; s < n_seqs; ++s) {
+      const int n = (q_start[s + 1] - q_start[s] + QT - 1) / QT;
+      if (tile < n) break;
+      tile -= n;
+    }
+    if (s >= n_seqs) return;
+    const int q_len = q_start[s + 1] - q_start[s];
+    const int first = tile * QT;
+    const int npos = min(QT, q_len - first);
+    const int nrows = npos * G;
+    if (wave * 32 >= nrows) return;                // (no barrier follows: waves are on their own)
+    const int pos0 = ctx_len[s] - q_len + first;
+    const int row = wave * 32 + c;
+    row_ok = row < nrows;
+    const int qi = row_ok ? row / G : 0;
+    h = kvh * G + (row_ok ? row % G : 0);
+    tok = q_start[s] + first + qi;
+    pos_r = pos0 + qi;
+    lo_r = (window > 0 && pos_r - window + 1 > 0) ? pos_r - window + 1 : 0;
+    const int p_lo = pos0 + (wave * 32) / G;                       // the wave's first position
+    const int p_hi = pos0 + (min(nrows, wave * 32 + 32) - 1) / G;  // and its last
+    k_first = (window > 0 && p_lo - window + 1 > 0) ? p_lo - window + 1 : 0;
+    k_end = p_hi + 1;
+  }
   const int* table = block_table + (size_t)s * max_pages;
-  const bool row_ok = c < G;
-  const int h = kvh * G + (row_ok ? c : 0);
 
   ta_bf16x8_t qf[HD / 16];
   {
-    const bf16_t* qrow = q + (size_t)s * q_stride + (size_t)h * HD;
+    const bf16_t* qrow = q + (size_t)tok * q_stride + (size_t)h * HD;
 #pragma unroll
     for (int i = 0; i < HD / 16; ++i) {
       ta_u32x4_t v = {0u, 0u, 0u, 0u};
@@ -480,8 +525,15 @@ __global__ __launch_bounds__(256) void tied_attention_decode_kernel(
   const bool has_sink = sink && split == 0;
   float m = has_sink ? 0.f : -INFINITY, l = has_sink ? 1.f : 0.f;
 
-  const int k_begin = k_first / TA_KEYS * TA_KEYS + split * wave_keys;
-  const int k_end = min(pos + 1, k_begin + wave_keys);
+  int k_begin = k_first / TA_KEYS * TA_KEYS;
+  if constexpr (DECODE) {
+    k_begin += split * wave_keys;
+    k_end = min(k_end, k_begin + wave_keys);
+  } else if (n_splits > 1) {
+    const int share = (k_end - k_begin + n_splits * TA_KEYS - 1) / (n_splits * TA_KEYS) * TA_KEYS;
+    k_begin += split * share;
+    k_end = min(k_end, k_begin + share);
+  }
 
   // this lane's key of a chunk: key base + c, values 16 i + 8 hl .. + 8 of it for every i
   ta_u32x4_t kf[HD / 16], kn[HD / 16];
@@ -506,8 +558,7 @@ __global__ __launch_bounds__(256) void tied_attention_decode_kernel(
 #pragma unroll
     for (int i = 0; i < HD / 16; ++i)
       sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const ta_bf16x8_t*)&kf[i], qf[i], sc, 0, 0, 0);
-    // the chunk transposed into the wave's tile (the reads of the chunk before are done: they
-    // fed MFMAs whose results were used below)
+    // the chunk transposed into the wave's tile
 #pragma unroll
     for (int i = 0; i < HD / 16; ++i) {
       const bf16_t* e = (const bf16_t*)&kf[i];
@@ -516,12 +567,23 @@ __global__ __launch_bounds__(256) void tied_attention_decode_kernel(
         kt[(16 * i + 8 * hl + x) * LDT + ta_swz(c, 16 * i + 8 * hl)] = e[x];
     }
     float cmax = -INFINITY;
+    // a chunk that every row of the wave sees whole needs no mask
+    const bool whole = row_ok && base >= lo_r && base + TA_KEYS - 1 <= pos_r &&
+                       base >= k_first && base + TA_KEYS <= k_end;
+    if (__all(whole)) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int key = base + 8 * (r / 4) + 4 * hl + r % 4;
-      const bool seen = row_ok && key >= k_first && key < k_end;
-      sc[r] = seen ? sc[r] * scale_log2 : -INFINITY;
-      cmax = fmaxf(cmax, sc[r]);
+      for (int r = 0; r < 16; ++r) {
+        sc[r] *= scale_log2;
+        cmax = fmaxf(cmax, sc[r]);
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = base + 8 * (r / 4) + 4 * hl + r % 4;
+        const bool seen = row_ok && key >= lo_r && key <= pos_r && key >= k_first && key < k_end;
+        sc[r] = seen ? sc[r] * scale_log2 : -INFINITY;
+        cmax = fmaxf(cmax, sc[r]);
+      }
     }
     cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));
     const float m_new = fmaxf(m, cmax);
@@ -536,10 +598,12 @@ __global__ __launch_bounds__(256) void tied_attention_decode_kernel(
     psum += __shfl_xor(psum, 32, 64);
     l = l * corr + psum;
     m = m_new;
+    if (__any(corr != 1.0f)) {
 #pragma unroll
-    for (int i = 0; i < HD / 32; ++i)
+      for (int i = 0; i < HD / 32; ++i)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][r] *= corr;
+        for (int r = 0; r < 16; ++r) acc[i][r] *= corr;
+    }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();               // the wave's transposed tile is written
 #pragma unroll
@@ -569,25 +633,46 @@ __global__ __launch_bounds__(256) void tied_attention_decode_kernel(
     for (int i = 0; i < HD / 16; ++i) kf[i] = kn[i];
   }
   if (!row_ok) return;
-  const size_t slot = ((size_t)s * nH + h) * n_splits + split;
-  float* po = ws_o + slot * HD;
+  // acc[i][r] is element d = 32 i + 8 (r / 4) + 4 hl + r % 4 of this lane's row
+  if (DECODE || n_splits > 1) {
+    const size_t slot = ((size_t)tok * nH + h) * n_splits + split;
+    float* po = ws_o + slot * HD;
 #pragma unroll
-  for (int i = 0; i < HD / 32; ++i)
+    for (int i = 0; i < HD / 32; ++i)
 #pragma unroll
-    for (int r4 = 0; r4 < 4; ++r4)
-      *(float4*)(po + 32 * i + 8 * r4 + 4 * hl) = make_float4(acc[i][4 * r4], acc[i][4 * r4 + 1],
-                                                              acc[i][4 * r4 + 2], acc[i][4 * r4 + 3]);
-  if (hl == 0) {
-    ws_ml[2 * slot] = m;
-    ws_ml[2 * slot + 1] = l;
+      for (int r4 = 0; r4 < 4; ++r4)
+        *(float4*)(po + 32 * i + 8 * r4 + 4 * hl) = make_float4(acc[i][4 * r4], acc[i][4 * r4 + 1],
+                                                                acc[i][4 * r4 + 2], acc[i][4 * r4 + 3]);
+    if (hl == 0) {
+      ws_ml[2 * slot] = m;
+      ws_ml[2 * slot + 1] = l;
+    }
+  } else {
+    const float inv = 1.0f / l;
+    bf16_t* orow = out + ((size_t)tok * nH + h) * HD;
+    const bf16_t* grow = gate != nullptr ? gate + (size_t)tok * gate_stride + (size_t)h * HD : nullptr;
+#pragma unroll
+    for (int i = 0; i < HD / 32; ++i)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const int d = 32 * i + 8 * r4 + 4 * hl;
+        float v[4];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+          v[x] = acc[i][4 * r4 + x] * inv;
+          if (grow != nullptr) v[x] *= 1.0f / (1.0f + expf(-bf16_to_float(grow[d + x])));
+        }
+        *(uint2*)(orow + d) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+      }
   }
 }
 
-#define TA_DEC_LAUNCH(HD)                                                                        \
+#define TA_WAVE_LAUNCH(HD, DEC)                                                                   \
   case HD:                                                                                       \
-    hipLaunchKernelGGL(tied_attention_decode_kernel<HD>, grid, dim3(256), 0, stream,             \
-                       (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, block_table, ctx_len,  \
-                       ws_o, ws_ml, scale, window, sink, nH, nKV, page_size, max_pages,          \
+    hipLaunchKernelGGL((tied_attention_wave_kernel<HD, DEC>), grid, dim3(256), 0, stream,        \
+                       (const bf16_t*)q, q_stride, (const bf16_t*)gate, gate_stride,             \
+                       (const bf16_t*)k_pool, block_table, q_start, ctx_len, (bf16_t*)out, ws_o, \
+                       ws_ml, scale, window, sink, n_seqs, nH, nKV, page_size, max_pages, QT,    \
                        wave_keys);                                                               \
     break;
 
@@ -680,12 +765,45 @@ extern "C" int zf_tied_attention_decode(const void* q, long long q_stride, const
       4 * n_blocks > ZF_WAVE || wave_keys <= 0 || wave_keys % TA_KEYS != 0 || !ws_o || !ws_ml)
     return -2;
   dim3 grid(n_seqs, nKV, n_blocks);
+  const int* q_start = nullptr;
+  const int QT = 1;
   switch (hd) {
-    TA_DEC_LAUNCH(32) TA_DEC_LAUNCH(64) TA_DEC_LAUNCH(96) TA_DEC_LAUNCH(128)
+    TA_WAVE_LAUNCH(32, true) TA_WAVE_LAUNCH(64, true) TA_WAVE_LAUNCH(96, true)
+    TA_WAVE_LAUNCH(128, true)
     default: return -3;
   }
   hipLaunchKernelGGL(tied_attention_merge_kernel, dim3(n_seqs, nH), dim3(ZF_WAVE), 0, stream,
                      ws_o, ws_ml, (const bf16_t*)gate, gate_stride, (bf16_t*)out, nH, hd,
                      4 * n_blocks);
+  ZF_CHECK_LAUNCH();
+}
+
+// Prompt portions by the same waves-on-their-own scheme: a workgroup's four waves take 32 rows
+// each of a tile of 128 / G positions and walk their own keys (no barrier; the keys a
+// workgroup's waves share come to each through the caches).  Head sizes up to 128, at most 32
+// query heads a kv head.  n_tiles as for zf_tied_attention_mfma.  n_splits > 1: every wave's
+// keys in that many parts, the partial results in ws_o / ws_ml (as above) and merged.
+extern "C" int zf_tied_attention_rows(const void* q, long long q_stride, const void* gate,
+                                      long long gate_stride, const void* k_pool,
+                                      const int* block_table, const int* q_start,
+                                      const int* ctx_len, void* out, float* ws_o, float* ws_ml,
+                                      float scale, int window, int sink, int T, int n_seqs,
+                                      int n_tiles, int nH, int nKV, int hd, int page_size,
+                                      int max_pages, int n_splits, hipStream_t stream) {
+  if (T <= 0 || n_tiles <= 0) return 0;
+  if (nKV <= 0 || nH % nKV != 0 || nH / nKV > 32 || page_size <= 0 || n_splits < 1 ||
+      n_splits > ZF_WAVE || (n_splits > 1 && (!ws_o || !ws_ml)))
+    return -2;
+  const int QT = TA_ROWS / (nH / nKV);
+  dim3 grid(n_tiles, nKV, n_splits);
+  const int wave_keys = 0;
+  switch (hd) {
+    TA_WAVE_LAUNCH(32, false) TA_WAVE_LAUNCH(64, false) TA_WAVE_LAUNCH(96, false)
+    TA_WAVE_LAUNCH(128, false)
+    default: return -3;
+  }
+  if (n_splits > 1)
+    hipLaunchKernelGGL(tied_attention_merge_kernel, dim3(T, nH), dim3(ZF_WAVE), 0, stream, ws_o,
+                       ws_ml, (const bf16_t*)gate, gate_stride, (bf16_t*)out, nH, hd, n_splits);
   ZF_CHECK_LAUNCH();
 }

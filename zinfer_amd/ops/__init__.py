@@ -1522,6 +1522,8 @@ TIED_MFMA_HEAD_DIMS = (32, 64, 96, 128, 192, 256)
 TIED_MFMA_ROWS = 128          # (position, head) pairs a workgroup of the MFMA kernel takes
 TIED_SPLIT_KEYS = 256         # least keys a split of a decode step's context holds
 TIED_SPLIT_WORKGROUPS = 512   # splits are made until about this many workgroups run
+TIED_ROWS_WAVES = 2048        # a prompt portion's keys are cut in parts until this many waves run
+TIED_ROWS_MAX_PARTS = 4
 TIED_DECODE_WORKGROUPS = 1024  # the same for the decode kernel (whose every wave is a split)
 
 
@@ -1549,14 +1551,16 @@ def tied_attention(q, gate, k_pool, block_table, q_start, ctx_len, seq_index, ou
 @_launches("attention")
 def tied_attention_mfma(q, gate, k_pool, block_table, q_start, ctx_len, out, scale, window, sink,
                         n_heads, n_kv_heads, head_dim, page_size, max_q_len, max_ctx_len,
-                        n_splits: Optional[int] = None) -> None:
+                        n_splits: Optional[int] = None, shared_tiles: Optional[bool] = None) -> None:
     """The bfloat16 MFMA form of ``shared_kv_attention`` (see there for the arguments).  Scores
     and the soft-max are 32-bit; a weight enters the second product as the sum of two bfloat16
     numbers.  A step in which every sequence brings one token runs the decode kernel (head
     sizes up to 128, at most 32 heads a kv head): each context is split over ``n_splits``
     workgroups of four waves that are splits of their own (None: by the block table's width and
     the window, never by the contexts themselves, so that a captured step replays for other
-    contexts), and the partial results are merged."""
+    contexts), and the partial results are merged.  Prompt portions of those shapes run the
+    same waves-on-their-own scheme, a wave per 32 (position, head) rows; ``shared_tiles`` True
+    (and every other shape) runs the kernel whose workgroup stages the keys once for 128 rows."""
     for t in (q, gate, k_pool, block_table, q_start, ctx_len, out):
         if t is not None and not t.is_cuda:
             raise KernelUnavailable("the HIP kernels run on GPU tensors only")
@@ -1585,7 +1589,7 @@ def tied_attention_mfma(q, gate, k_pool, block_table, q_start, ctx_len, out, sca
     G = n_heads // n_kv_heads
     lib = build.load("sink_attention")
     keys = max_pages * page_size if window <= 0 else min(max_pages * page_size, window)
-    if max_q_len == 1 and T == n_seqs and head_dim <= 128 and G <= 32:
+    if max_q_len == 1 and T == n_seqs and head_dim <= 128 and G <= 32 and not shared_tiles:
         # a decode step: every wave of a workgroup is a split of its own
         # (``tied_attention_decode_kernel``); about 1024 workgroups, at least 64 keys a wave
         span = keys + 31                      # the first chunk starts at a multiple of 32
@@ -1606,6 +1610,33 @@ def tied_attention_mfma(q, gate, k_pool, block_table, q_start, ctx_len, out, sca
         return
     QT = max(1, TIED_MFMA_ROWS // G)
     n_tiles = (T + QT - 1) // QT + n_seqs
+    if shared_tiles is None:
+        shared_tiles = not (head_dim <= 128 and G <= 32)
+    if not shared_tiles:
+        # prompt portions: every wave walks the keys of its own 32 rows
+        if head_dim > 128 or G > 32:
+            raise KernelUnavailable("tied_attention_mfma: waves on their own take head sizes up "
+                                    "to 128 and 32 heads a kv head")
+        # few waves behind long contexts: every wave's keys in parts, so that the last rows of
+        # a prompt do not run alone at the end and a SIMD holds more than one wave
+        parts = n_splits
+        if parts is None:
+            waves = (T * n_heads + 31) // 32
+            parts = 1
+            while parts < TIED_ROWS_MAX_PARTS and waves * parts < TIED_ROWS_WAVES \
+                    and min(keys, max_ctx_len) >= 256 * parts:
+                parts *= 2
+        ws_o = ws_ml = None
+        if parts > 1:
+            ws_o = _workspace("tied_o", T * n_heads * parts * head_dim, torch.float32, q.device)
+            ws_ml = _workspace("tied_ml", T * n_heads * parts * 2, torch.float32, q.device)
+        _check(lib.zf_tied_attention_rows(
+            _ptr(q), ctypes.c_longlong(qs), _ptr(gate), ctypes.c_longlong(gs), _ptr(k_pool),
+            _ptr(block_table), _ptr(q_start), _ptr(ctx_len), _ptr(out), _ptr(ws_o), _ptr(ws_ml),
+            ctypes.c_float(scale), int(window), 1 if sink else 0, T, n_seqs, n_tiles, n_heads,
+            n_kv_heads, head_dim, page_size, max_pages, parts, _stream()),
+            "tied_attention_mfma (rows)")
+        return
     if n_splits is None:
         n_splits = 1
         if max_q_len == 1 and n_seqs * n_kv_heads < 256:
