@@ -47,6 +47,24 @@ def test_norm_rows_store_and_add(T, W, centred, bias):
     assert rel_err(acc, base.double() + ref) < tol(torch.float32)
 
 
+@pytest.mark.parametrize("T, W", [(1, 48), (7, 336), (3, 4096), (2, 8192)])
+@pytest.mark.parametrize("dt", DTYPES)
+def test_norm_add_norm_is_the_two_norms_one_after_the_other(T, W, dt):
+    y, x = _rand((T, W), 81, 2.0) + 0.5, _rand((T, W), 82)
+    wa, ba = 1 + _rand((W,), 83, 0.2), _rand((W,), 84, 0.5)
+    wb, bb = 1 + _rand((W,), 85, 0.2), _rand((W,), 86, 0.5)
+    dev = lambda t: t.to(DEV)
+    x1, out1 = dev(x), torch.empty((T, W), dtype=dt, device=DEV)
+    ops.norm_add_norm(dev(y), dev(wa), dev(ba), 1e-5, True, x1, dev(wb), dev(bb), 1e-6, True, out1)
+    x2, out2 = dev(x), torch.empty((T, W), dtype=dt, device=DEV)
+    ops.norm_rows(dev(y), dev(wa), dev(ba), 1e-5, x2, True, add=True)
+    ops.norm_rows(x2, dev(wb), dev(bb), 1e-6, out2, True)
+    assert rel_err(x1, x2) < 1e-6 and rel_err(out1, out2.double()) < (1e-6 if dt == torch.float32 else 2.0 ** -8)
+    ref_x = x.double() + P.layer_norm(y, wa, ba, 1e-5)
+    assert rel_err(x1, ref_x) < 2e-5
+    assert rel_err(out1, P.layer_norm(ref_x, wb, bb, 1e-6)) < tol(dt)
+
+
 def test_layer_norm_of_a_row_with_a_large_mean():
     """The variance comes from the deviations: a mean a thousand times the spread leaves it."""
     x = 1000.0 + _rand((4, 256), 5, 1.0)

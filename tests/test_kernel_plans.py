@@ -145,7 +145,7 @@ TESTED_AGAINST = {
     "stream_read": "test_kernels_gpu.py:test_stream_read_reads_every_byte_once",
     "mfma_loop": "test_kernels_gpu.py:test_mfma_loop_sums_its_products",
     "check_tables": "test_kernels_gpu.py:test_check_tables_reports_and_never_traps",
-    "norm_rows": "plain_fezupel.py:layer_norm",
+    "norm_rows": "plain_fezupel.py:layer_norm", "norm_add_norm": "plain_fezupel.py:layer_norm",
     "embed_position": "test_fezupel_kernels_gpu.py:test_embed_position",
     "kv_rows_write": "test_fezupel_kernels_gpu.py:test_attention_against_plain",
     "shared_kv_attention": "plain_fezupel.py:sink_window_attention",

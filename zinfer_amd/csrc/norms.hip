@@ -125,6 +125,101 @@ extern "C" int zf_norm_rows(const float* x, const float* gain, const float* bias
   ZF_CHECK_LAUNCH();
 }
 
+// ---------------------------------------------------------------- a norm behind a sublayer and the one before the next
+// x += norm_a(y); out = norm_b(x): the norm that closes a sublayer adds its result into the
+// residual stream, and the norm that opens the next sublayer reads the sum while the row is
+// still in registers (one kernel and one pass over the stream instead of two).  Widths that
+// are a multiple of 4 up to 8192.  Each norm as in norm_rows (32-bit, mean first, variance from
+// the deviations): the same numbers as the two kernels one after the other.
+template <typename TO>
+__global__ __launch_bounds__(256) void norm_add_norm_kernel(
+    const float* __restrict__ y, const float* __restrict__ gain_a, const float* __restrict__ bias_a,
+    float eps_a, int centred_a, float* __restrict__ x, const float* __restrict__ gain_b,
+    const float* __restrict__ bias_b, float eps_b, int centred_b, TO* __restrict__ out, int W) {
+  __shared__ float red[16];
+  const float4* yrow = (const float4*)(y + (size_t)blockIdx.x * W);
+  float4* xrow = (float4*)(x + (size_t)blockIdx.x * W);
+  TO* o = out + (size_t)blockIdx.x * W;
+  const int n4 = W / 4;
+  float4 v[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int c = threadIdx.x + i * 256;
+    v[i] = c < n4 ? yrow[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  // one norm over the row held in v: v = (v - mean) * inv * gain + bias, in place
+  auto norm = [&](const float* gain, const float* bias, float eps, int centred) {
+    float mean = 0.f;
+    if (centred) {
+      float s = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+      mean = block_sum(s, red) / (float)W;
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int c = threadIdx.x + i * 256;
+      if (c < n4) {
+        v[i].x -= mean; v[i].y -= mean; v[i].z -= mean; v[i].w -= mean;
+        ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+      }
+    }
+    ss = block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)W + eps);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int c = threadIdx.x + i * 256;
+      if (c < n4) {
+        const float4 g = ((const float4*)gain)[c];
+        float4 b = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (bias != nullptr) b = ((const float4*)bias)[c];
+        v[i].x = v[i].x * inv * g.x + b.x;
+        v[i].y = v[i].y * inv * g.y + b.y;
+        v[i].z = v[i].z * inv * g.z + b.z;
+        v[i].w = v[i].w * inv * g.w + b.w;
+      }
+    }
+  };
+  norm(gain_a, bias_a, eps_a, centred_a);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int c = threadIdx.x + i * 256;
+    if (c < n4) {
+      const float4 r = xrow[c];
+      v[i].x = r.x + v[i].x; v[i].y = r.y + v[i].y; v[i].z = r.z + v[i].z; v[i].w = r.w + v[i].w;
+      xrow[c] = v[i];
+    }
+  }
+  norm(gain_b, bias_b, eps_b, centred_b);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int c = threadIdx.x + i * 256;
+    if (c < n4) {
+      store_from_float<TO>(o + 4 * c + 0, v[i].x);
+      store_from_float<TO>(o + 4 * c + 1, v[i].y);
+      store_from_float<TO>(o + 4 * c + 2, v[i].z);
+      store_from_float<TO>(o + 4 * c + 3, v[i].w);
+    }
+  }
+}
+
+extern "C" int zf_norm_add_norm(const float* y, const float* gain_a, const float* bias_a,
+                                float eps_a, int centred_a, float* x, const float* gain_b,
+                                const float* bias_b, float eps_b, int centred_b, void* out,
+                                int out_dtype, int T, int W, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (W <= 0 || W % 4 != 0 || W > 8192) return -2;
+  if (out_dtype == ZF_F32)
+    hipLaunchKernelGGL(norm_add_norm_kernel<float>, dim3(T), dim3(256), 0, stream, y, gain_a,
+                       bias_a, eps_a, centred_a, x, gain_b, bias_b, eps_b, centred_b, (float*)out, W);
+  else
+    hipLaunchKernelGGL(norm_add_norm_kernel<bf16_t>, dim3(T), dim3(256), 0, stream, y, gain_a,
+                       bias_a, eps_a, centred_a, x, gain_b, bias_b, eps_b, centred_b,
+                       (bf16_t*)out, W);
+  ZF_CHECK_LAUNCH();
+}
+
 // ---------------------------------------------------------------- embedding plus a learned position
 // x[t, :] = E[id[t], :] * scale + P[position[t], :], widened to float32
 template <typename TW>

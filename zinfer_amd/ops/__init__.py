@@ -1424,6 +1424,37 @@ def norm_rows(x: torch.Tensor, gain: torch.Tensor, bias: Optional[torch.Tensor],
                             _stream()), "norm_rows")
 
 
+NORM_ADD_NORM_MAX_WIDTH = 8192
+
+
+def norm_add_norm_covers(width: int) -> bool:
+    return width % 4 == 0 and 0 < width <= NORM_ADD_NORM_MAX_WIDTH
+
+
+@_launches("norm_rope_write")
+def norm_add_norm(y: torch.Tensor, gain_a, bias_a, eps_a: float, centred_a: bool,
+                  x: torch.Tensor, gain_b, bias_b, eps_b: float, centred_b: bool,
+                  out: torch.Tensor) -> None:
+    """x += norm_a(y); out = norm_b(x), row by row in 32-bit (``norm_rows`` with ``add`` and then
+    ``norm_rows``, in one kernel, the same numbers): the norm behind a sublayer and the norm
+    before the next one.  ``y`` and ``x`` float32 [T, W], W a multiple of 4 up to 8192."""
+    _need_gpu(y, gain_a, bias_a, x, gain_b, bias_b, out)
+    T, W = x.shape
+    vecs = [v for v in (gain_a, bias_a, gain_b, bias_b) if v is not None]
+    if y.shape != x.shape or out.shape != x.shape or y.dtype != torch.float32 \
+            or x.dtype != torch.float32 or gain_a is None or gain_b is None \
+            or any(v.dtype != torch.float32 or v.shape != (W,) for v in vecs) \
+            or not norm_add_norm_covers(W):
+        raise KernelUnavailable(f"norm_add_norm: float32 rows {tuple(y.shape)} and "
+                                f"{tuple(x.shape)}, float32 [W] gains and biases, W a multiple "
+                                f"of 4 up to {NORM_ADD_NORM_MAX_WIDTH}")
+    lib = build.load("norms")
+    _check(lib.zf_norm_add_norm(_ptr(y), _ptr(gain_a), _ptr(bias_a), ctypes.c_float(eps_a),
+                                1 if centred_a else 0, _ptr(x), _ptr(gain_b), _ptr(bias_b),
+                                ctypes.c_float(eps_b), 1 if centred_b else 0, _ptr(out), _dt(out),
+                                T, W, _stream()), "norm_add_norm")
+
+
 @_launches("other")
 def embed_position(table: torch.Tensor, ids: torch.Tensor, pos_table: torch.Tensor,
                    positions: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:

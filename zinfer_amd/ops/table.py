@@ -9,7 +9,7 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Callable, Dict
 
-from . import (gated_act, moe_grouped, tied_attention_mfma)
+from . import (gated_act, moe_grouped, norm_add_norm, tied_attention_mfma)
 from . import (embed_position, kv_rows_write, moe_down, moe_gate_up, moe_route, norm_rows,
                shared_kv_attention)
 from . import (advance_decode, apply_penalties, argmax, argmax_no_alloc, cast, check_tables,
@@ -68,6 +68,8 @@ KERNELS: Dict[str, KernelEntry] = {
                                "own: the read stream bandwidths are measured against"),
     "norm_rows": KernelEntry(norm_rows, "norms", "own: layer norm / RMS norm with a bias, stored "
                              "or added to the stream"),
+    "norm_add_norm": KernelEntry(norm_add_norm, "norms", "own: the norm behind a sublayer, the "
+                                 "residual sum and the norm before the next sublayer"),
     "embed_position": KernelEntry(embed_position, "norms", "own: embedding plus a learned "
                                   "position row"),
     "kv_rows_write": KernelEntry(kv_rows_write, "sink_attention", "own: key rows into pages"),

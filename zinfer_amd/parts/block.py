@@ -95,7 +95,9 @@ class SandwichNormBlock(Block):
                                            prefix + spec.ff_post_norm_prefix)
             self.parts += [self.ff_norm, self.feed_forward, self.ff_post_norm]
         self.parts = tuple(self.parts)
-        self.entry_norm = None          # nothing a sum into the stream could leave for it
+        # the norm that reads the stream first: the block before may already have run it, in
+        # the kernel of its own last norm (``NormedRows`` in ``step.norm_ready``)
+        self.entry_norm = self.mixer_norm
         self.graph_safe = all(p.graph_safe for p in self.parts)
         self.kernel_modules = tuple(sorted({m for p in self.parts for m in p.kernel_modules}))
 
@@ -118,23 +120,56 @@ class SandwichNormBlock(Block):
     def hint_providers(self):
         return [q for p in self.parts for q in p.hint_providers()]
 
-    def _sublayer(self, norm, part, post, x, step, *cache) -> None:
-        step.norm_ready = step.norm_after = None
-        h = norm.forward(x, step.scratch("normed", x.shape, self.ctx.act_dtype))
+    def _sublayer(self, norm, part, post, x, step, args, then, ready):
+        """One sublayer; ``args``: what the part takes behind the step (a mixer its cache).
+        ``ready``: the rows ``norm`` would give, if whoever summed into the
+        stream last has run it already.  ``then``: the norm that reads the stream next; if the
+        closing norm's kernel can run it too, its rows come back (else None)."""
+        if ready is not None:
+            h = ready
+        else:
+            h = norm.forward(x, step.scratch("normed", x.shape, self.ctx.act_dtype))
         branch = step.scratch("branch", x.shape, torch.float32)
         if getattr(part, "stores_output", False):
-            part.forward(h, branch, step, *cache, accumulate=False)
+            part.forward(h, branch, step, *args, accumulate=False)
         else:
             branch.zero_()
-            part.forward(h, branch, step, *cache)
+            part.forward(h, branch, step, *args)
         step.norm_ready = None
+        fused = getattr(post, "forward_add_then", None)
+        if then is not None and fused is not None:
+            # (the mixer or feed-forward is done with the buffer its input lay in)
+            out = step.scratch("normed", x.shape, self.ctx.act_dtype)
+            if fused(branch, x, then, out):
+                return out
         post.forward_add(branch, x)
+        return None
 
     def forward(self, x, step, cache) -> None:
-        self._sublayer(self.mixer_norm, self.mixer, self.mixer_post_norm, x, step, cache)
+        after_block = step.norm_after_block
+        left, step.norm_ready, step.norm_after = step.norm_ready, None, None
+        ready = left.normed if isinstance(left, NormedRows) and left.fits(self.mixer_norm, x) \
+            else None
+        then = self.ff_norm if self.feed_forward is not None else after_block
+        h = self._sublayer(self.mixer_norm, self.mixer, self.mixer_post_norm, x, step,
+                           (cache,), then, ready)
         if self.feed_forward is not None:
-            self._sublayer(self.ff_norm, self.feed_forward, self.ff_post_norm, x, step)
+            h = self._sublayer(self.ff_norm, self.feed_forward, self.ff_post_norm, x, step, (),
+                               after_block, h)
         step.norm_after = None
+        # what the next block's first norm would compute is there already
+        step.norm_ready = NormedRows(after_block, x, h) if h is not None else None
+
+
+class NormedRows:
+    """The rows ``normed`` = ``norm(x)`` that a block's last kernel already made for the norm
+    that reads the stream next."""
+
+    def __init__(self, norm, x: torch.Tensor, normed: torch.Tensor):
+        self.norm, self.x, self.normed = norm, x, normed
+
+    def fits(self, norm, x: torch.Tensor) -> bool:
+        return self.norm is norm and self.x.data_ptr() == x.data_ptr() and self.x.shape == x.shape
 
 
 register_part("block", PreNormBlockSpec, PreNormBlock)

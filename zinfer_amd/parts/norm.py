@@ -155,6 +155,18 @@ class LayerNorm(Norm):
         ops.norm_rows(x, self.gain, self.bias, float(self.spec.eps), residual,
                       bool(self.spec.centred), add=True)
 
+    def forward_add_then(self, x: torch.Tensor, residual: torch.Tensor, then: "Norm",
+                         out: torch.Tensor) -> bool:
+        """residual += norm(x) and out = then(residual) in one kernel, if ``then`` is a norm of
+        this kind and the width allows; False (and nothing done) otherwise."""
+        if not isinstance(then, LayerNorm) or not residual.is_cuda \
+                or not ops.norm_add_norm_covers(residual.shape[1]):
+            return False
+        ops.norm_add_norm(x, self.gain, self.bias, float(self.spec.eps), bool(self.spec.centred),
+                          residual, then.gain, then.bias, float(then.spec.eps),
+                          bool(then.spec.centred), out)
+        return True
+
 
 register_part("norm", RmsNormSpec, RmsNorm)
 register_part("norm", LayerNormSpec, LayerNorm)
