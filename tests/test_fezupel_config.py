@@ -120,3 +120,18 @@ def test_plain_layer_pieces():
     q = torch.zeros((1, 4)); k = torch.tensor([[2.0, 4.0, 6.0, 8.0]])
     o = plain_fezupel.sink_window_attention(q, k, 1, 1, 4, 1.0, 3)
     assert torch.allclose(o, k.double() / 2)
+
+
+def test_command_line_writes_and_inspects_a_model_folder(tmp_path, capsys):
+    from zinfer_amd.cli import main
+    cfg = tmp_path / "config.json"
+    cfg.write_text(json.dumps(fz.FZ_B))
+    out = str(tmp_path / "m")
+    assert main(["random-model", str(cfg), out, "--seed", "4", "--dtype", "float32"]) == 0
+    assert main(["inspect-config", out]) == 0
+    text = capsys.readouterr().out
+    assert "architecture: Fezupel" in text and "width: 72" in text and "model_type: fezupel" in text
+    assert text.count("architecture:") == 1
+    assert main(["inspect-weights", out]) == 0
+    text = capsys.readouterr().out
+    assert "tensor l0.mlp.router.b: dtype=F32 shape=[3] " in text

@@ -218,3 +218,24 @@ def test_replay_program_on_a_model_folder(tmp_path):
         outputs = {st["step"]: np.fromfile(os.path.join(out, f"{st['step']}.f32"), dtype="<f4")
                    for st in steps if any(e["want"] for e in st["entries"])}
         _compare(steps, outputs, ref, fz.CONFIGS[name]["vocab"], dtype, name)
+
+
+def test_generation_through_the_command_line(tmp_path):
+    """``bin/zinfer generate-token-ids`` on a Fezupel folder: the oracle's greedy tokens."""
+    name = "A"
+    path = _write_folder(name, str(tmp_path / name), torch.float32)
+    prompt = fz.tokens(11, fz.CONFIGS[name]["vocab"], 9)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "zinfer"), "generate-token-ids",
+                        path, ",".join(map(str, prompt)), "6", "--dtype", "float32"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    line = [l for l in r.stdout.splitlines() if l.startswith("tokens: ")][0]
+    got = json.loads(line[len("tokens: "):])
+    assert got[:len(prompt)] == prompt and len(got) == len(prompt) + 6
+    w = fz.weights_of(name)
+    logits = P.forward(fz.CONFIGS[name], w, got[:-1])
+    for i in range(len(prompt) - 1, len(got) - 1):
+        top2 = torch.topk(logits[i], 2).values
+        if float(top2[0] - top2[1]) > 1e-3 * float(logits[i].abs().max()):
+            assert int(logits[i].argmax()) == got[i + 1]

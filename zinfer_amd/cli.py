@@ -283,7 +283,7 @@ def cmd_inspect_config(args: List[str]) -> int:
     # every key of the typed configuration, whatever the architecture; numbers as the
     # reference prints them (theta as an integer, eps in scientific notation)
     for key, value in cfg.to_dict().items():
-        if key in ("model_type", "architectures"):
+        if key in ("model_type", "architectures", "architecture"):
             continue
         if isinstance(value, bool):
             value = str(value).lower()

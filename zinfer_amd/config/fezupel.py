@@ -158,6 +158,10 @@ class FezupelConfig:
     def vocab_size(self) -> int:
         return self.vocab
 
+    @property
+    def model_type(self) -> str:
+        return "fezupel"
+
     # ------------------------------------------------------------------ the model's parts
     def layer_order(self) -> Tuple[int, ...]:
         n = len(self.layers)
