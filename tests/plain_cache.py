@@ -35,11 +35,13 @@ class PlainPool:
 
 
 class PlainCache:
-    """``windows[g]``: the window of group g (None: every key is kept)."""
+    """``windows[g]``: the window of group g (None: every key is kept); ``chunks[g]``: the
+    chunk of group g (None: no chunks): a query reads only keys of its own chunk."""
 
     def __init__(self, windows: Sequence[Optional[int]], page_size: int, num_pages: int,
-                 max_requests: int):
+                 max_requests: int, chunks: Optional[Sequence[Optional[int]]] = None):
         self.windows = list(windows)
+        self.chunks = list(chunks) if chunks is not None else [None] * len(self.windows)
         self.ps = page_size
         self.pools = [PlainPool(num_pages) for _ in windows]
         self.slots = PlainPool(max_requests)
@@ -49,8 +51,11 @@ class PlainCache:
         return (tokens + self.ps - 1) // self.ps
 
     def _first_needed(self, g: int, length: int) -> int:
-        w = self.windows[g]
-        return 0 if w is None else max(0, length - w + 1) // self.ps
+        w, c = self.windows[g], self.chunks[g]
+        first = 0 if w is None else max(0, length - w + 1)
+        if c is not None:
+            first = max(first, length // c * c)
+        return first // self.ps
 
     def _missing(self, g: int, table: List[int], length: int, new_len: int) -> int:
         last = self._pages_for(new_len)
@@ -105,7 +110,7 @@ class PlainCache:
         r = self.requests[rid]
         r["length"] = new_len
         for g, w in enumerate(self.windows):
-            if w is None:
+            if w is None and self.chunks[g] is None:
                 continue
             table = r["tables"][g]
             gone = [i for i in range(min(self._first_needed(g, new_len), len(table)))

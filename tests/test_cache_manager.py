@@ -141,8 +141,8 @@ def test_random_orders_lose_nothing(seed, window):
 @pytest.mark.parametrize("seed", range(6))
 def test_native_bookkeeping_follows_the_plain_model(seed):
     """The native core against a plain model in lists and dicts, call by call under a random
-    order of calls (requests that come, grow in portions, are cut back, end; two groups, one
-    with a window; few pages, so that they run out and are used again): the same block tables
+    order of calls (requests that come, grow in portions, are cut back, end; three groups, one
+    with a window, one whose queries read their own chunk of positions only; few pages, so that they run out and are used again): the same block tables
     page for page, the same free pages and slots, the same answers to what is missing and
     what fits, the same refusals; and the step tables the core packs are the tables' pages."""
     import numpy as np
@@ -150,9 +150,11 @@ def test_native_bookkeeping_follows_the_plain_model(seed):
     rng = random.Random(100 + seed)
     ps, num_pages, max_requests = rng.choice([2, 4, 16]), rng.choice([6, 9, 14]), 3
     window = rng.choice([3, 7, 20])
-    needs = [KVNeed(1, 4), KVNeed(1, 4, window)]
-    m = CacheManager(needs, [None, None], ps, num_pages, max_requests, torch.float32, "cpu")
-    plain = PlainCache([None, window], ps, num_pages, max_requests)
+    chunk = rng.choice([1, 5, 8, 19])
+    needs = [KVNeed(1, 4), KVNeed(1, 4, window), KVNeed(1, 4, chunk=chunk)]
+    m = CacheManager(needs, [None, None, None], ps, num_pages, max_requests, torch.float32, "cpu")
+    plain = PlainCache([None, window, None], ps, num_pages, max_requests,
+                       chunks=[None, None, chunk])
     names = ["a", "b", "c", "d", "e"]
     packed = 0
     for _ in range(600):
@@ -188,16 +190,18 @@ def test_native_bookkeeping_follows_the_plain_model(seed):
             plain.commit(rid, new_len)
         for r, rec in plain.requests.items():
             assert m.length(r) == rec["length"] and m.state_slot(r) == rec["slot"]
-            for g in range(2):
+            for g in range(3):
                 assert m.table(g, r) == rec["tables"][g], (op, rid, r, g)
         assert m.num_free_pages() == [len(p.free_list) for p in plain.pools]
         assert m.num_free_slots() == len(plain.slots.free_list)
         assert [g.pages.handed_out for g in m.groups] == [p.handed_out for p in plain.pools]
         m.check()
         # a step of the live requests that hold something: one more token each
-        step = [r for r in plain.requests if plain.requests[r]["length"] > 0]
-        if step and all(m.pages_missing(r, m.length(r) + 1) == [0, 0] for r in step):
-            for g in range(2):
+        # (of a chunk that has just ended the last token's page may have gone back already)
+        step = [r for r, rec in plain.requests.items() if rec["length"] > 0
+                and rec["tables"][2][(rec["length"] - 1) // ps] != NO_PAGE]
+        if step and all(m.pages_missing(r, m.length(r) + 1) == [0, 0, 0] for r in step):
+            for g in range(3):
                 starts = [m.length(r) - 1 for r in step]       # the last token held, again
                 width = max(len(plain.requests[r]["tables"][g]) for r in step) + 1
                 table = np.empty((len(step), width), dtype=np.int32)

@@ -109,6 +109,9 @@ class CacheManager:
         if not self._core:
             raise ValueError(f"a cache of {num_pages} pages of {page_size} tokens for "
                              f"{max_requests} requests cannot be made")
+        for g, need in enumerate(by_need):
+            if need.chunk is not None:
+                self._raise(self._lib.zc_set_chunk(self._core, g, int(need.chunk)))
         self._where: Dict[int, Tuple[int, int]] = {}     # schedule position -> (group, run)
         for need, runs in by_need.items():
             g = len(self.groups)
@@ -223,6 +226,8 @@ class CacheManager:
             n = n_tokens
             if grp.need.window is not None:
                 n = min(n, grp.need.window + portion + self.page_size)
+            if grp.need.chunk is not None:
+                n = min(n, grp.need.chunk + portion + self.page_size)
             out.append((n + self.page_size - 1) // self.page_size)
         return out
 

@@ -22,6 +22,7 @@ def core_lib() -> ctypes.CDLL:
         lib.zc_last_error.restype = ctypes.c_char_p
         for name, restype, argtypes in (
                 ("zc_create", vp, (i32, pi32, i32, i32, i32)), ("zc_destroy", None, (vp,)),
+                ("zc_set_chunk", i32, (vp, i32, i32)),
                 ("zc_has_request", i32, (vp, i64)), ("zc_length", i32, (vp, i64, pi32)),
                 ("zc_state_slot", i32, (vp, i64, pi32)), ("zc_add_request", i32, (vp, i64, pi32)),
                 ("zc_pages_missing", None, (vp, i64, i32, pi32)),

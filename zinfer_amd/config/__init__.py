@@ -3,7 +3,10 @@ from .registry import (ArchitectureEntry, TextHooks, entry_for, load_config, rea
                        unregister_architecture)
 from .specs import (GatedExpertSpec, LayerNormSpec, MoeSpec, SandwichNormBlockSpec,
                     TiedKeyValueAttentionSpec)
+from .specs import (DenseMlpSpec, LatentAttentionSpec, LeadingRotarySpec, MaskedGqaAttentionSpec,
+                    PostNormBlockSpec)
 from .specs import (GqaAttentionSpec, ModelSpec, NoPositionSpec, PreNormBlockSpec, RmsNormSpec,
                     RotaryHalfSplitSpec, ScheduleEntry, SwiGluSpec)
 from .qwen3 import Qwen3Config
 from .fezupel import FezupelConfig
+from .lodenex import LodenexConfig

@@ -81,6 +81,97 @@ class TiedKeyValueAttentionSpec:
 
 
 @dataclass(frozen=True)
+class LeadingRotarySpec:
+    """Rotation of the first ``dims`` elements of a head (the rest pass unchanged) in the pairs
+    (i, i + dims/2) by the angle position * frequencies[i]; cosine and sine are multiplied by
+    ``magnitude``.  The frequencies are plain data, so that any rule for them (a base alone,
+    wavelengths slowed beyond a length, a ramp between two turn counts) gives the same part;
+    ``config.rotary`` holds the rules.  There is no table of positions: the angle is formed
+    from the position where it is used, in 32-bit."""
+    dims: int
+    frequencies: Tuple[float, ...]
+    magnitude: float = 1.0
+
+
+@dataclass(frozen=True)
+class MaskedGqaAttentionSpec:
+    """Causal grouped-query attention with separate key and value sizes and these options:
+    ``qk_norm_eps``: an RMS norm over the whole q projection and one over the whole k projection
+    (all heads at once) with gains of those sizes, before the rotation; ``rotary``: a
+    ``LeadingRotarySpec`` or None; ``softcap``: scores become cap * tanh(score / cap);
+    ``window`` (the last ``window`` positions) and ``chunk`` (only keys of the query's own
+    chunk of that many positions, counted from position 0); ``sink``: one learned number a head
+    whose exponential joins the soft-max's denominator; ``head_gate``: head h's output is
+    multiplied by sigmoid(W_g h)_h, one number a head.  The ``*_name`` fields are the tensor
+    names below the mixer's prefix."""
+    hidden_size: int
+    n_heads: int
+    n_kv_heads: int
+    head_dim: int
+    value_dim: int
+    scale: float
+    qk_norm_eps: Optional[float] = None
+    rotary: Optional[LeadingRotarySpec] = None
+    softcap: Optional[float] = None
+    window: Optional[int] = None
+    chunk: Optional[int] = None
+    sink: bool = False
+    head_gate: bool = False
+    q_name: str = "q_proj.weight"
+    k_name: str = "k_proj.weight"
+    v_name: str = "v_proj.weight"
+    o_name: str = "o_proj.weight"
+    q_norm_name: str = "q_norm.weight"
+    k_norm_name: str = "k_norm.weight"
+    sink_name: str = "sinks"
+    gate_name: str = "g_proj.weight"
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Attention whose keys and values come from one latent row a token: q = W_uq N(W_dq h)
+    laid out head by head as [head_dim plain | rot_dim rotated]; W_dkv h = [latent of kv_rank,
+    normed | rot_dim, not normed, rotated: one key part shared by all heads]; per head the
+    plain key is W_uk latent and the value W_uv latent; the score is scale * (q_plain . k_plain
+    + q_rot . k_rot).  The cache holds the latent and the rotated part only.  ``window`` /
+    ``chunk`` as in ``MaskedGqaAttentionSpec``; ``element_gate``: the concatenated heads are
+    multiplied by sigmoid(W_g h) before the output projection."""
+    hidden_size: int
+    n_heads: int
+    head_dim: int
+    rot_dim: int
+    value_dim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    norm_eps: float
+    rotary: Optional[LeadingRotarySpec] = None
+    window: Optional[int] = None
+    chunk: Optional[int] = None
+    element_gate: bool = False
+    dq_name: str = "q_a_proj.weight"
+    dq_norm_name: str = "q_a_layernorm.weight"
+    uq_name: str = "q_b_proj.weight"
+    dkv_name: str = "kv_a_proj_with_mqa.weight"
+    dkv_norm_name: str = "kv_a_layernorm.weight"
+    uk_name: str = "k_b_proj.weight"
+    uv_name: str = "v_b_proj.weight"
+    gate_name: str = "g_proj.weight"
+    o_name: str = "o_proj.weight"
+
+
+@dataclass(frozen=True)
+class DenseMlpSpec:
+    """down(act(up(x))), no gate: ``activation`` is "gelu" (the exact form with erf),
+    "gelu_tanh" or "silu"."""
+    hidden_size: int
+    intermediate_size: int
+    activation: str = "gelu"
+    up_name: str = "up_proj.weight"
+    down_name: str = "down_proj.weight"
+
+
+@dataclass(frozen=True)
 class GatedExpertSpec:
     """down(act(gate(x), up(x))) with g = min(gate, limit), u = clamp(up, -limit, limit)
     (``limit`` None: neither is clamped) and act = g * sigmoid(alpha * g) * (u + shift)."""
@@ -149,6 +240,21 @@ class SandwichNormBlockSpec:
     mixer_norm_prefix: str = "input_layernorm."
     mixer_post_norm_prefix: str = "post_attention_layernorm."
     ff_norm_prefix: str = "pre_feedforward_layernorm."
+    ff_post_norm_prefix: str = "post_feedforward_layernorm."
+
+
+@dataclass(frozen=True)
+class PostNormBlockSpec:
+    """x += norm1(mixer(x)); x += norm2(ff(x)): the sublayers read the stream as it is, and the
+    only norms stand behind them, ahead of the residual sums.  ``feed_forward`` None: the layer
+    is its first line (and declares no ``ff_post_norm``)."""
+    mixer: object
+    feed_forward: Optional[object]
+    mixer_post_norm: object
+    ff_post_norm: Optional[object] = None
+    mixer_prefix: str = "self_attn."
+    ff_prefix: str = "mlp."
+    mixer_post_norm_prefix: str = "post_attention_layernorm."
     ff_post_norm_prefix: str = "post_feedforward_layernorm."
 
 

@@ -497,6 +497,39 @@ extern "C" int zf_swiglu(const void* gu, void* out, int dtype, int T, int I,
   ZF_CHECK_LAUNCH();
 }
 
+// ---------------------------------------------------------------- an activation alone, in place or not
+// kind 0: gelu(z) = z/2 (1 + erf(z / sqrt 2));  kind 1: its tanh form
+// z/2 (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)));  kind 2: silu(z) = z / (1 + exp(-z)).
+// 32-bit arithmetic on values of either storage type.
+__device__ __forceinline__ float activation_value(float z, int kind) {
+  if (kind == 0) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752440f));
+  if (kind == 1)
+    return 0.5f * z * (1.0f + tanhf(0.79788456080286535588f * (z + 0.044715f * z * z * z)));
+  return z / (1.0f + expf(-z));
+}
+
+template <typename T>
+__global__ void activation_kernel(const T* __restrict__ x, T* __restrict__ out, size_t n,
+                                  int kind) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n) return;
+  store_from_float<T>(out + idx, activation_value(load_as_float<T>(x + idx), kind));
+}
+
+extern "C" int zf_activation(const void* x, void* out, int dtype, long long n, int kind,
+                             hipStream_t stream) {
+  if (n <= 0) return 0;
+  if (kind < 0 || kind > 2) return -2;
+  const unsigned blocks = (unsigned)((n + 255) / 256);
+  if (dtype == ZF_F32)
+    hipLaunchKernelGGL(activation_kernel<float>, dim3(blocks), dim3(256), 0, stream,
+                       (const float*)x, (float*)out, (size_t)n, kind);
+  else
+    hipLaunchKernelGGL(activation_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream,
+                       (const bf16_t*)x, (bf16_t*)out, (size_t)n, kind);
+  ZF_CHECK_LAUNCH();
+}
+
 // ---------------------------------------------------------------- cast and poison
 // out[i] = in[i] in the other storage type (bfloat16 -> float32 is exact, float32 -> bfloat16
 // rounds to nearest even): weights stored in one type for a build in the other are converted

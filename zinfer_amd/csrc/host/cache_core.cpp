@@ -82,6 +82,7 @@ struct Request {
 
 struct Group {
   int window;      // -1: every key is kept
+  int chunk = -1;  // > 0: a query reads only keys of its own chunk of this many positions
   PagePool pages;
   std::vector<int> freed;      // what the last call gave back, in the order it was freed
   Group(int w, int n) : window(w), pages(n) {}
@@ -99,12 +100,15 @@ struct Core {
   int pages_for(int tokens) const { return (tokens + page_size - 1) / page_size; }
   // logical index of the first page a query at position >= length can still read
   int first_needed(const Group& g, int length) const {
-    if (g.window < 0) return 0;
-    return std::max(0, length - g.window + 1) / page_size;
+    int first = 0;                                   // a position, then its page
+    if (g.window >= 0) first = std::max(first, length - g.window + 1);
+    if (g.chunk > 0) first = std::max(first, length / g.chunk * g.chunk);
+    return first / page_size;
   }
+  static bool keeps_all(const Group& g) { return g.window < 0 && g.chunk <= 0; }
   int missing(const Group& g, const std::vector<int>& table, int length, int new_len) const {
     const int last = pages_for(new_len);
-    if (g.window < 0) return std::max(0, last - (int)table.size());      // no holes
+    if (keeps_all(g)) return std::max(0, last - (int)table.size());      // no holes
     int n = 0;
     for (int i = first_needed(g, length); i < last; ++i)
       if (i >= (int)table.size() || table[(size_t)i] == NO_PAGE) ++n;
@@ -145,6 +149,15 @@ void* zc_create(int n_groups, const int* windows, int page_size, int num_pages, 
   Core* c = new Core(page_size, max_requests);
   for (int g = 0; g < n_groups; ++g) c->groups.emplace_back(windows[g], num_pages);
   return c;
+}
+// a group whose queries read only the keys of their own chunk of `chunk` positions (counted
+// from position 0) gives the pages of earlier chunks back; set before any request is added
+int zc_set_chunk(void* h, int group, int chunk) {
+  Core* c = (Core*)h;
+  if (group < 0 || group >= (int)c->groups.size() || chunk < 1 || !c->requests.empty())
+    return fail(BAD, "zc_set_chunk: a group of the core, a chunk of at least 1, no live request");
+  c->groups[(size_t)group].chunk = chunk;
+  return OK;
 }
 void zc_destroy(void* h) { delete (Core*)h; }
 
@@ -236,7 +249,7 @@ int zc_commit(void* h, long long rid, int new_len) {
   r.length = new_len;
   for (size_t g = 0; g < c->groups.size(); ++g) {
     Group& grp = c->groups[g];
-    if (grp.window < 0) continue;
+    if (Core::keeps_all(grp)) continue;
     std::vector<int>& table = r.tables[g];
     const int first = std::min(c->first_needed(grp, new_len), (int)table.size());
     std::vector<int> gone;

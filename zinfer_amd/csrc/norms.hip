@@ -220,6 +220,80 @@ extern "C" int zf_norm_add_norm(const float* y, const float* gain_a, const float
   ZF_CHECK_LAUNCH();
 }
 
+// ---------------------------------------------------------------- a norm behind a sublayer, and the sum as the next one reads it
+// x += norm(y); out = x in out's storage type: for blocks whose sublayers read the stream as it
+// is (no norm in front of them), the kernel that closes one sublayer leaves the sum in the
+// type the next sublayer's products take.  Widths that are a multiple of 4 up to 8192; the
+// norm as in norm_rows, the same numbers.
+template <typename TO>
+__global__ __launch_bounds__(256) void norm_add_store_kernel(
+    const float* __restrict__ y, const float* __restrict__ gain, const float* __restrict__ bias,
+    float eps, int centred, float* __restrict__ x, TO* __restrict__ out, int W) {
+  __shared__ float red[16];
+  const float4* yrow = (const float4*)(y + (size_t)blockIdx.x * W);
+  float4* xrow = (float4*)(x + (size_t)blockIdx.x * W);
+  TO* o = out + (size_t)blockIdx.x * W;
+  const int n4 = W / 4;
+  float4 v[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int c = threadIdx.x + i * 256;
+    v[i] = c < n4 ? yrow[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  float mean = 0.f;
+  if (centred) {
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+    mean = block_sum(s, red) / (float)W;
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int c = threadIdx.x + i * 256;
+    if (c < n4) {
+      v[i].x -= mean; v[i].y -= mean; v[i].z -= mean; v[i].w -= mean;
+      ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+    }
+  }
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)W + eps);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int c = threadIdx.x + i * 256;
+    if (c < n4) {
+      const float4 g = ((const float4*)gain)[c];
+      float4 b = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (bias != nullptr) b = ((const float4*)bias)[c];
+      const float4 r = xrow[c];
+      float4 s;
+      s.x = r.x + (v[i].x * inv * g.x + b.x);
+      s.y = r.y + (v[i].y * inv * g.y + b.y);
+      s.z = r.z + (v[i].z * inv * g.z + b.z);
+      s.w = r.w + (v[i].w * inv * g.w + b.w);
+      xrow[c] = s;
+      store_from_float<TO>(o + 4 * c + 0, s.x);
+      store_from_float<TO>(o + 4 * c + 1, s.y);
+      store_from_float<TO>(o + 4 * c + 2, s.z);
+      store_from_float<TO>(o + 4 * c + 3, s.w);
+    }
+  }
+}
+
+extern "C" int zf_norm_add_store(const float* y, const float* gain, const float* bias, float eps,
+                                 int centred, float* x, void* out, int out_dtype, int T, int W,
+                                 hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (W <= 0 || W % 4 != 0 || W > 8192) return -2;
+  if (out_dtype == ZF_F32)
+    hipLaunchKernelGGL(norm_add_store_kernel<float>, dim3(T), dim3(256), 0, stream, y, gain, bias,
+                       eps, centred, x, (float*)out, W);
+  else
+    hipLaunchKernelGGL(norm_add_store_kernel<bf16_t>, dim3(T), dim3(256), 0, stream, y, gain,
+                       bias, eps, centred, x, (bf16_t*)out, W);
+  ZF_CHECK_LAUNCH();
+}
+
 // ---------------------------------------------------------------- embedding plus a learned position
 // x[t, :] = E[id[t], :] * scale + P[position[t], :], widened to float32
 template <typename TW>

@@ -1883,3 +1883,231 @@ def sample_topk(logits: torch.Tensor, params: torch.Tensor, out: torch.Tensor) -
     lib = build.load("sampling")
     _check(lib.zf_sample_topk(_ptr(logits), _ptr(params), _ptr(out), n, V, _stream()),
            "sample_topk")
+
+
+# ------------------------------------------------------------------------- an activation alone
+ACTIVATIONS = {"gelu": 0, "gelu_tanh": 1, "silu": 2}
+
+
+@_launches("norm_rope_write")
+def activation(x: torch.Tensor, out: torch.Tensor, kind: str) -> None:
+    """out = act(x) element by element, in 32-bit on values of either storage type: "gelu"
+    (the exact form with erf), "gelu_tanh", "silu".  ``out`` may be ``x``."""
+    _need_gpu(x, out)
+    if x.shape != out.shape or x.dtype != out.dtype or kind not in ACTIVATIONS:
+        raise KernelUnavailable(f"activation: {tuple(x.shape)} {x.dtype} -> {tuple(out.shape)} "
+                                f"{out.dtype}, kind {kind!r} of {sorted(ACTIVATIONS)}")
+    lib = build.load("elementwise")
+    _check(lib.zf_activation(_ptr(x), _ptr(out), _dt(x), ctypes.c_longlong(x.numel()),
+                             ACTIVATIONS[kind], _stream()), "activation")
+
+
+@_launches("norm_rope_write")
+def norm_add_store(y: torch.Tensor, gain: torch.Tensor, bias: Optional[torch.Tensor], eps: float,
+                   centred: bool, x: torch.Tensor, out: torch.Tensor) -> None:
+    """x += norm(y); out = x rounded to ``out``'s type, row by row in 32-bit (``norm_rows`` with
+    ``add`` and a cast, in one kernel, the same numbers).  ``y`` and ``x`` float32 [T, W], W a
+    multiple of 4 up to 8192."""
+    _need_gpu(y, gain, bias, x, out)
+    T, W = x.shape
+    if y.shape != x.shape or out.shape != x.shape or y.dtype != torch.float32 \
+            or x.dtype != torch.float32 or gain.dtype != torch.float32 or gain.shape != (W,) \
+            or (bias is not None and (bias.dtype != torch.float32 or bias.shape != (W,))) \
+            or not norm_add_norm_covers(W):
+        raise KernelUnavailable(f"norm_add_store: float32 rows {tuple(y.shape)} and "
+                                f"{tuple(x.shape)}, float32 [W] gain and bias, W a multiple of 4 "
+                                f"up to {NORM_ADD_NORM_MAX_WIDTH}")
+    lib = build.load("norms")
+    _check(lib.zf_norm_add_store(_ptr(y), _ptr(gain), _ptr(bias), ctypes.c_float(eps),
+                                 1 if centred else 0, _ptr(x), _ptr(out), _dt(out), T, W,
+                                 _stream()), "norm_add_store")
+
+
+# ------------------------------------------------------------------------- attention with a cap, a sink, chunks or a window, a gate
+class RowSegment:
+    """Columns [src_off, src_off + width) of a projection's rows and what happens to them on the
+    way out (``project_rows``): ``gain`` [width] float32: an RMS norm over the whole segment with
+    ``eps``; the segment is ``width / hd`` heads, of each the elements [rot_off, rot_off +
+    rot_dims) are rotated by the token's position in the pairs (i, i + rot_dims / 2) with the
+    angles position * ``freq`` [rot_dims / 2] (float32), cosine and sine times ``mag``; the
+    elements of a head below ``skip`` are not written.  The rest goes to ``dst``: plain rows
+    [T, ...] where head h starts at column dst_off + h * dst_hd (dst_hd None: hd - skip), or
+    (``pool_heads`` given) a pool [page, kv head, row, dst_hd] at the token's slot, from column
+    dst_off of the pool row on."""
+
+    def __init__(self, src_off: int, width: int, dst: torch.Tensor, *, gain=None, eps: float = 0.0,
+                 hd: Optional[int] = None, rot_off: int = 0, rot_dims: int = 0, freq=None,
+                 mag: float = 1.0, skip: int = 0, dst_off: int = 0, dst_hd: Optional[int] = None,
+                 pool_heads: Optional[int] = None):
+        self.src_off, self.width, self.dst = int(src_off), int(width), dst
+        self.gain, self.eps = gain, float(eps)
+        self.hd = int(hd) if hd is not None else int(width)
+        self.rot_off, self.rot_dims, self.freq, self.mag = int(rot_off), int(rot_dims), freq, float(mag)
+        self.skip, self.dst_off = int(skip), int(dst_off)
+        self.dst_hd = int(dst_hd) if dst_hd is not None else self.hd - self.skip
+        self.pool_heads = pool_heads
+
+
+PROJECT_ROWS_MAX_SEGMENTS = 4
+
+
+@_launches("norm_rope_write")
+def project_rows(src: torch.Tensor, positions: torch.Tensor, slot_mapping: Optional[torch.Tensor],
+                 page_size: int, segments) -> None:
+    """Every row of ``src`` [T, C] (contiguous rows, any row stride), segment by segment as
+    ``RowSegment`` says: norm, rotation by ``positions`` [T], then into rows or pages.  All
+    arithmetic is 32-bit; a row's result depends on that row and its position alone."""
+    for t in (src, positions, slot_mapping):
+        if t is not None and not t.is_cuda:
+            raise KernelUnavailable("the HIP kernels run on GPU tensors only")
+    _i32(positions, "positions")
+    T, C = src.shape
+    stride = _columns(src, "project_rows: src")
+    n = len(segments)
+    if not 0 < n <= PROJECT_ROWS_MAX_SEGMENTS or positions.shape[0] != T:
+        raise KernelUnavailable(f"project_rows: 1 to {PROJECT_ROWS_MAX_SEGMENTS} segments and a "
+                                "position a row")
+    ints, floats, ptrs, strides = [], [], [], []
+    for g in segments:
+        pool = g.pool_heads is not None
+        ok = 0 <= g.src_off and g.src_off + g.width <= C and g.width > 0 and g.hd > 0 \
+            and g.width % g.hd == 0 and g.rot_dims % 2 == 0 and 0 <= g.rot_off \
+            and g.rot_off + g.rot_dims <= g.hd and 0 <= g.skip < g.hd \
+            and g.dst.is_cuda and g.dst.dtype == src.dtype and g.dst_off >= 0 \
+            and (g.gain is None or (g.gain.is_cuda and g.gain.dtype == torch.float32
+                                    and g.gain.shape == (g.width,) and g.gain.is_contiguous())) \
+            and (g.rot_dims == 0 or (g.freq is not None and g.freq.is_cuda
+                                     and g.freq.dtype == torch.float32
+                                     and g.freq.shape == (g.rot_dims // 2,)))
+        heads = g.width // max(g.hd, 1)
+        if ok and pool:
+            _i32(slot_mapping, "slot_mapping")
+            ok = slot_mapping.shape[0] == T and g.dst.is_contiguous() and heads == g.pool_heads \
+                and g.dst_off + g.hd - g.skip <= g.dst_hd \
+                and g.dst.numel() % (g.pool_heads * page_size * g.dst_hd) == 0
+            strides.append(0)
+        elif ok:
+            ok = g.dst.dim() == 2 and g.dst.stride(1) == 1 and g.dst.shape[0] == T \
+                and g.dst_off + (heads - 1) * g.dst_hd + g.hd - g.skip <= g.dst.shape[1]
+            strides.append(g.dst.stride(0) if ok else 0)
+        if not ok:
+            raise KernelUnavailable(f"project_rows: a segment of columns {g.src_off}.."
+                                    f"{g.src_off + g.width} (heads of {g.hd}) does not fit its "
+                                    f"source {tuple(src.shape)} or destination "
+                                    f"{tuple(g.dst.shape)} {g.dst.dtype}")
+        ints += [g.src_off, g.width, g.hd, g.rot_off, g.rot_dims, g.skip, 1 if pool else 0,
+                 g.dst_off, g.dst_hd, g.pool_heads or 0, 0]
+        floats += [g.eps, g.mag]
+        ptrs += [g.gain.data_ptr() if g.gain is not None else None,
+                 g.freq.data_ptr() if g.rot_dims else None, g.dst.data_ptr()]
+    lib = build.load("masked_attention")
+    _check(lib.zf_project_rows(
+        _ptr(src), _dt(src), ctypes.c_longlong(stride), _ptr(positions), _ptr(slot_mapping), T,
+        int(page_size), n, (ctypes.c_int * len(ints))(*ints),
+        (ctypes.c_float * len(floats))(*floats), (ctypes.c_void_p * len(ptrs))(*ptrs),
+        (ctypes.c_longlong * len(strides))(*strides), _stream()), "project_rows")
+
+
+GATE_MODES = {None: 0, "element": 1, "head": 2}
+
+
+def _masked_attention_checks(what, q, gate, gate_mode, k_pool, v_pool, sink, block_table, q_start,
+                             ctx_len, seq_index, out, n_heads, n_kv_heads, key_width,
+                             value_width, page_size, max_ctx_len):
+    for t in (q, gate, k_pool, v_pool, sink, block_table, q_start, ctx_len, seq_index, out):
+        if t is not None and not t.is_cuda:
+            raise KernelUnavailable("the HIP kernels run on GPU tensors only")
+    T = q.shape[0]
+    if gate_mode not in GATE_MODES or (gate_mode is None) != (gate is None):
+        raise KernelUnavailable(f"{what}: gate mode {gate_mode!r} of {list(GATE_MODES)}, with a "
+                                "gate exactly when there is a mode")
+    gate_cols = {None: 0, "element": n_heads * value_width, "head": n_heads}[gate_mode]
+    if q.shape[1] != n_heads * key_width or out.shape != (T, n_heads * value_width) \
+            or not out.is_contiguous() or out.dtype != q.dtype or k_pool.dtype != q.dtype \
+            or (v_pool is not None and v_pool.dtype != q.dtype) \
+            or (gate is not None and (gate.shape != (T, gate_cols) or gate.dtype != q.dtype)) \
+            or (sink is not None and (sink.dtype != torch.float32 or sink.shape != (n_heads,))):
+        raise KernelUnavailable(f"{what}: q [T, nH * key width], out [T, nH * value width], the "
+                                "gate [T, nH * value width] or [T, nH], all of the pools' dtype; "
+                                "the sink float32 [nH]")
+    for t, name in ((block_table, "block_table"), (q_start, "q_start"), (ctx_len, "ctx_len"),
+                    (seq_index, "seq_index")):
+        _i32(t, name)
+    if n_kv_heads <= 0 or n_heads % n_kv_heads != 0:
+        raise KernelUnavailable(f"{what}: InvalidGrouping")
+    if key_width < 1 or not 0 < value_width <= MAX_HEAD_DIM \
+            or (v_pool is None and value_width > key_width):
+        raise KernelUnavailable(f"{what}: key rows of {key_width}, value rows of {value_width} "
+                                f"(1..{MAX_HEAD_DIM}; without a value pool at most the key's)")
+    if max_ctx_len > block_table.shape[1] * page_size:
+        raise KernelUnavailable(f"{what}: block table shorter than the context")
+    n_seqs = ctx_len.shape[0]
+    if q_start.shape[0] != n_seqs + 1 or block_table.shape[0] != n_seqs \
+            or seq_index.shape[0] != T or not block_table.is_contiguous() \
+            or not k_pool.is_contiguous() or (v_pool is not None and not v_pool.is_contiguous()):
+        raise KernelUnavailable(f"{what}: per-sequence arrays disagree in length")
+
+
+@_launches("attention")
+def masked_attention(q: torch.Tensor, gate: Optional[torch.Tensor], gate_mode: Optional[str],
+                     k_pool: torch.Tensor, v_pool: Optional[torch.Tensor],
+                     sink: Optional[torch.Tensor], block_table, q_start, ctx_len, seq_index,
+                     out: torch.Tensor, scale: float, cap: float, window: int, chunk: int,
+                     n_heads: int, n_kv_heads: int, key_width: int, value_width: int,
+                     page_size: int, max_ctx_len: int) -> None:
+    """Causal grouped-query attention over paged pools: keys [page, kv head, row, key width],
+    values [page, kv head, row, value width], or with ``v_pool`` None the first ``value_width``
+    columns of the key rows.  Token t of sequence s = seq_index[t] has position p = ctx_len[s] -
+    q_len[s] + (t - q_start[s]) and reads the keys j <= p with p - j < window (window > 0) and
+    floor(j / chunk) == floor(p / chunk) (chunk > 0).  Scores are scale * q . k, then with
+    cap > 0 cap * tanh(score / cap).  ``sink`` [nH] float32: the soft-max's denominator holds
+    exp(sink_h) once more.  ``gate`` with mode "element" [T, nH * value width] or "head" [T, nH]:
+    the output is multiplied by sigmoid(gate).  ``q`` and ``gate`` may be column slices of a
+    wider product.  All arithmetic is 32-bit in both dtypes."""
+    _masked_attention_checks("masked_attention", q, gate, gate_mode, k_pool, v_pool, sink,
+                             block_table, q_start, ctx_len, seq_index, out, n_heads, n_kv_heads,
+                             key_width, value_width, page_size, max_ctx_len)
+    qs = _columns(q, "masked_attention: q")
+    gs = _columns(gate, "masked_attention: gate") if gate is not None else 0
+    lib = build.load("masked_attention")
+    code = lib.zf_masked_attention(
+        _ptr(q), ctypes.c_longlong(qs), _ptr(gate), ctypes.c_longlong(gs), GATE_MODES[gate_mode],
+        _ptr(k_pool), _ptr(v_pool), _dt(q), _ptr(sink), _ptr(block_table), _ptr(q_start),
+        _ptr(ctx_len), _ptr(seq_index), _ptr(out), ctypes.c_float(scale), ctypes.c_float(cap),
+        int(window), int(chunk), q.shape[0], n_heads, n_kv_heads, key_width, value_width,
+        page_size, block_table.shape[1], _stream())
+    if code == -3:
+        raise KernelUnavailable(f"masked_attention: key rows of {key_width} are wider than the "
+                                "kernel's staging area takes")
+    _check(code, "masked_attention")
+
+
+@_launches("products")
+def head_products(a: torch.Tensor, a_off: int, a_hd: int, w: torch.Tensor,
+                  gate: Optional[torch.Tensor], out: torch.Tensor, out_off: int,
+                  out_hd: int) -> None:
+    """A matrix a head: out[t, out_off + h * out_hd + n] = sum_k a[t, a_off + h * a_hd + k] *
+    w[h, n, k] for w [H, N, K], times sigmoid(gate[t, h * N + n]) if a gate is given.  ``a``,
+    ``out`` and ``gate`` are matrices with contiguous rows (any row stride).  32-bit sums in
+    ascending k whatever the dtypes: a row's result does not depend on the rows beside it."""
+    for t in (a, w, gate, out):
+        if t is not None and not t.is_cuda:
+            raise KernelUnavailable("the HIP kernels run on GPU tensors only")
+    T = a.shape[0]
+    if w.dim() != 3 or not w.is_contiguous():
+        raise KernelUnavailable("head_products: w must be [H, N, K], contiguous")
+    H, N, K = w.shape
+    a_stride = _columns(a, "head_products: a")
+    o_stride = _columns(out, "head_products: out")
+    g_stride = _columns(gate, "head_products: gate") if gate is not None else 0
+    if out.shape[0] != T or out.dtype != a.dtype or a_hd < K or out_hd < N or a_off < 0 \
+            or out_off < 0 or a_off + (H - 1) * a_hd + K > a.shape[1] \
+            or out_off + (H - 1) * out_hd + N > out.shape[1] \
+            or (gate is not None and (gate.shape != (T, H * N) or gate.dtype != a.dtype)):
+        raise KernelUnavailable(f"head_products: a {tuple(a.shape)}, w {tuple(w.shape)}, out "
+                                f"{tuple(out.shape)} do not fit together")
+    lib = build.load("masked_attention")
+    _check(lib.zf_head_products(
+        _ptr(a), _dt(a), ctypes.c_longlong(a_stride), int(a_off), int(a_hd), _ptr(w), _dt(w),
+        _ptr(gate), ctypes.c_longlong(g_stride), _ptr(out), ctypes.c_longlong(o_stride),
+        int(out_off), int(out_hd), T, H, N, K, _stream()), "head_products")

@@ -10,6 +10,7 @@ from dataclasses import dataclass
 from typing import Callable, Dict
 
 from . import (gated_act, moe_grouped, norm_add_norm, tied_attention_mfma)
+from . import (activation, head_products, masked_attention, norm_add_store, project_rows)
 from . import (embed_position, kv_rows_write, moe_down, moe_gate_up, moe_route, norm_rows,
                shared_kv_attention)
 from . import (advance_decode, apply_penalties, argmax, argmax_no_alloc, cast, check_tables,
@@ -84,6 +85,16 @@ KERNELS: Dict[str, KernelEntry] = {
     "moe_grouped": KernelEntry(moe_grouped, "moe", "own: the chosen experts over tokens sorted "
                                "by expert, MFMA tiles"),
     "gated_act": KernelEntry(gated_act, "moe", "own: the experts' activation alone"),
+    "activation": KernelEntry(activation, "elementwise", "own: gelu (erf or tanh form) or silu "
+                              "alone"),
+    "norm_add_store": KernelEntry(norm_add_store, "norms", "own: the norm behind a sublayer, the "
+                                  "residual sum, and the sum in the products' type"),
+    "project_rows": KernelEntry(project_rows, "masked_attention", "own: a projection's rows "
+                                "normed over whole segments, rotated in part, into rows or pages"),
+    "masked_attention": KernelEntry(masked_attention, "masked_attention", "own: attention with a "
+                                    "score cap, a learned sink, chunks or a window, a gate; the "
+                                    "values a pool or the keys' leading columns"),
+    "head_products": KernelEntry(head_products, "masked_attention", "own: a matrix a head"),
     "mfma_loop": KernelEntry(mfma_loop, "gemm",
                              "own: MFMAs alone, the rate the tiled products are measured against"),
 }

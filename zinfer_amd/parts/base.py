@@ -48,7 +48,9 @@ class TensorDecl:
 @dataclass(frozen=True)
 class KVNeed:
     """A cache of keys and values that grows with the context; with ``window`` only the
-    last ``window`` positions are ever read, so earlier pages may be given back.  A key row
+    last ``window`` positions are ever read, and with ``chunk`` only the positions of the
+    query's own chunk of that many (counted from position 0), so earlier pages may be given
+    back.  A key row
     is ``head_dim`` wide; a value row ``value_dim`` (None: as wide as a key), so a mixer whose
     values are narrower or wider than its keys (or that keeps one shared latent row:
     ``n_kv_heads`` 1) gets pools of its own widths; ``value_dim`` 0: the values are the keys,
@@ -59,6 +61,7 @@ class KVNeed:
     window: Optional[int] = None
     value_dim: Optional[int] = None
     dtype: Optional[torch.dtype] = None
+    chunk: Optional[int] = None
 
     @property
     def key_width(self) -> int:

@@ -4,7 +4,7 @@ from typing import Dict
 
 import torch
 
-from ..config.specs import PreNormBlockSpec, SandwichNormBlockSpec
+from ..config.specs import PostNormBlockSpec, PreNormBlockSpec, SandwichNormBlockSpec
 from .base import Block, TensorDecl, build_part, register_part
 
 
@@ -172,5 +172,104 @@ class NormedRows:
         return self.norm is norm and self.x.data_ptr() == x.data_ptr() and self.x.shape == x.shape
 
 
+class StreamRows:
+    """The residual rows ``x`` in the activations' type, left by the kernel that last added
+    into them for a sublayer that reads the stream as it is."""
+
+    def __init__(self, x: torch.Tensor, rows: torch.Tensor):
+        self.x, self.rows = x, rows
+
+    def fits(self, x: torch.Tensor) -> bool:
+        return self.x.data_ptr() == x.data_ptr() and self.x.shape == x.shape
+
+
+class PostNormBlock(Block):
+    """x += norm1(mixer(x)); x += norm2(ff(x)): the sublayers read the stream itself, and each
+    one's output goes through a norm before it joins the stream.  A sublayer stores its output
+    in a float32 branch; the norm behind it reads the branch and adds its result to the stream
+    in 32-bit, and the same kernel leaves the sum in the type the next sublayer's products take
+    (``StreamRows``, handed across the layer's edge in ``step.norm_ready``).  In a 32-bit build
+    the sublayers read the stream's own rows.  Without a feed-forward the block is its first
+    line."""
+
+    def __init__(self, spec: PostNormBlockSpec, ctx, prefix):
+        super().__init__(spec, ctx, prefix)
+        self.mixer = build_part("mixer", spec.mixer, ctx, prefix + spec.mixer_prefix)
+        self.mixer_post_norm = build_part("norm", spec.mixer_post_norm, ctx,
+                                          prefix + spec.mixer_post_norm_prefix)
+        self.parts = [self.mixer, self.mixer_post_norm]
+        self.feed_forward = self.ff_post_norm = None
+        if spec.feed_forward is not None:
+            self.feed_forward = build_part("feed_forward", spec.feed_forward, ctx,
+                                           prefix + spec.ff_prefix)
+            self.ff_post_norm = build_part("norm", spec.ff_post_norm, ctx,
+                                           prefix + spec.ff_post_norm_prefix)
+            self.parts += [self.feed_forward, self.ff_post_norm]
+        self.parts = tuple(self.parts)
+        self.graph_safe = all(p.graph_safe for p in self.parts)
+        # (the cast of the stream's rows is the elementwise module's)
+        self.kernel_modules = tuple(sorted({"elementwise"}
+                                           | {m for p in self.parts for m in p.kernel_modules}))
+
+    def declare(self) -> Dict[str, TensorDecl]:
+        d: Dict[str, TensorDecl] = {}
+        for part in self.parts:
+            d.update(part.declare())
+        return d
+
+    def bind(self, tensors) -> None:
+        for part in self.parts:
+            part.bind(tensors)
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def accept_cache(self, cache) -> None:
+        self.mixer.accept_cache(cache)
+
+    def hint_providers(self):
+        return [q for p in self.parts for q in p.hint_providers()]
+
+    def _rows(self, x, step):
+        """The stream's rows as a sublayer's products take them."""
+        if self.ctx.act_dtype == torch.float32:
+            return x
+        from .. import ops
+        rows = step.scratch("stream_rows", x.shape, self.ctx.act_dtype)
+        ops.cast(x, rows)
+        return rows
+
+    def _sublayer(self, part, post, x, h, step, args):
+        """One sublayer on the rows ``h`` of the stream ``x``; returns the rows of the new
+        stream if the closing norm's kernel left them, else None."""
+        branch = step.scratch("branch", x.shape, torch.float32)
+        if getattr(part, "stores_output", False):
+            part.forward(h, branch, step, *args, accumulate=False)
+        else:
+            branch.zero_()
+            part.forward(h, branch, step, *args)
+        step.norm_ready = None
+        fused = getattr(post, "forward_add_store", None)
+        if self.ctx.act_dtype != torch.float32 and fused is not None:
+            # (the sublayer is done with the buffer its input lay in)
+            out = step.scratch("stream_rows", x.shape, self.ctx.act_dtype)
+            if fused(branch, x, out):
+                return out
+        post.forward_add(branch, x)
+        return None
+
+    def forward(self, x, step, cache) -> None:
+        left, step.norm_ready, step.norm_after = step.norm_ready, None, None
+        h = left.rows if isinstance(left, StreamRows) and left.fits(x) else self._rows(x, step)
+        h = self._sublayer(self.mixer, self.mixer_post_norm, x, h, step, (cache,))
+        if self.feed_forward is not None:
+            if h is None:
+                h = self._rows(x, step)
+            h = self._sublayer(self.feed_forward, self.ff_post_norm, x, h, step, ())
+        step.norm_after = None
+        step.norm_ready = StreamRows(x, h) if h is not None else None
+
+
+register_part("block", PostNormBlockSpec, PostNormBlock)
 register_part("block", PreNormBlockSpec, PreNormBlock)
 register_part("block", SandwichNormBlockSpec, SandwichNormBlock)

@@ -5,7 +5,7 @@ from typing import Dict
 import torch
 
 from .. import ops
-from ..config.specs import SwiGluSpec
+from ..config.specs import DenseMlpSpec, SwiGluSpec
 from .base import FeedForward, TensorDecl, register_part
 from .linear import Linear, place_matrix
 
@@ -68,4 +68,34 @@ class _probe:
         self.is_cuda, self.dtype, self.shape = g.is_cuda, g.dtype, (2 * g.shape[0], g.shape[1])
 
 
+class DenseMlp(FeedForward):
+    """d = W_down act(W_up m), no gate; the activation (``ops.ACTIVATIONS``) runs in 32-bit on
+    the product's values."""
+    graph_safe = True
+    stores_output = True
+    kernel_modules = ("elementwise", "gemm")
+
+    def declare(self) -> Dict[str, TensorDecl]:
+        s, p = self.spec, self.prefix
+        return {p + s.up_name: TensorDecl((s.intermediate_size, s.hidden_size)),
+                p + s.down_name: TensorDecl((s.hidden_size, s.intermediate_size))}
+
+    def bind(self, tensors) -> None:
+        s, p = self.spec, self.prefix
+        if s.activation not in ops.ACTIVATIONS:
+            from ..errors import ConfigError
+            raise ConfigError(f"activation {s.activation!r}: known are {sorted(ops.ACTIVATIONS)}")
+        self.up = Linear(place_matrix(tensors[p + s.up_name], self.ctx))
+        self.down = Linear(place_matrix(tensors[p + s.down_name], self.ctx))
+
+    def forward(self, h, residual, step, accumulate: bool = True) -> None:
+        if hasattr(h, "materialize"):
+            h = h.materialize()
+        a = step.scratch("ff_act", (h.shape[0], self.spec.intermediate_size), self.ctx.act_dtype)
+        self.up.forward(h, a)
+        ops.activation(a, a, self.spec.activation)
+        self.down.forward(a, residual, accumulate=accumulate, step=step if accumulate else None)
+
+
 register_part("feed_forward", SwiGluSpec, SwiGluMlp)
+register_part("feed_forward", DenseMlpSpec, DenseMlp)

@@ -155,6 +155,17 @@ class LayerNorm(Norm):
         ops.norm_rows(x, self.gain, self.bias, float(self.spec.eps), residual,
                       bool(self.spec.centred), add=True)
 
+    def forward_add_store(self, x: torch.Tensor, residual: torch.Tensor,
+                          out: torch.Tensor) -> bool:
+        """residual += norm(x) and out = residual in ``out``'s type in one kernel (for a block
+        whose next sublayer reads the stream as it is), if the width allows; False (and nothing
+        done) otherwise."""
+        if not residual.is_cuda or not ops.norm_add_norm_covers(residual.shape[1]):
+            return False
+        ops.norm_add_store(x, self.gain, self.bias, float(self.spec.eps),
+                           bool(self.spec.centred), residual, out)
+        return True
+
     def forward_add_then(self, x: torch.Tensor, residual: torch.Tensor, then: "Norm",
                          out: torch.Tensor) -> bool:
         """residual += norm(x) and out = then(residual) in one kernel, if ``then`` is a norm of
