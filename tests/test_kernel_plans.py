@@ -153,6 +153,10 @@ TESTED_AGAINST = {
     "moe_route": "plain_fezupel.py:route", "moe_gate_up": "plain_fezupel.py:clamped_expert",
     "moe_down": "plain_fezupel.py:clamped_expert", "moe_grouped": "plain_fezupel.py:clamped_expert",
     "gated_act": "test_fezupel_kernels_gpu.py:test_gated_act",
+    "activation": "plain_lodenex.py:gelu_erf", "norm_add_store": "plain_lodenex.py:rms_norm",
+    "project_rows": "plain_lodenex.py:rotate_leading",
+    "masked_attention": "plain_lodenex.py:masked_softmax_values",
+    "head_products": "test_lodenex_kernels_gpu.py:test_head_products",
 }
 
 

@@ -1,0 +1,263 @@
+"""Lodenex models through the engine against ``plain_lodenex``, in 32-bit and in bfloat16:
+whole prompts; most of a prompt and then its last tokens one by one; portions of changing
+size down to two tokens; token by token from the first token on (long decoding: many times
+the chunks and windows); mixed batches of four live requests in a pool so small that pages are
+used again (what was given back is overwritten with NaN first); the same bits however a prompt
+is cut in 32-bit; greedy generation through the entry point and the scheduler; the replay
+program and the command line on a model folder."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import lodenex_tiny as lx
+import plain_lodenex as P
+import traces
+from gpu_util import DEV
+
+pytestmark = pytest.mark.gpu
+
+# float32: what is left is the order of sums and the 32-bit angles.  bfloat16: activations are
+# rounded to 8 bits of mantissa some ten times a layer against the same bfloat16-rounded
+# weights, and the norm behind every sublayer brings each branch back to full size, so the
+# error of a layer does not shrink with its output: about 0.004 of the largest logit a layer at
+# the median, three to four times that at the worst position.
+TOL = {"float32": 4e-5, "bfloat16": 0.03}
+LENGTHS = {"A": (1, 5, 23, 60, 150), "B": (2, 9, 47, 130), "C": (3, 17, 64), "D": (4, 33, 100, 260)}
+_ref = {}
+
+
+def _tol(name, dtype):
+    return TOL[dtype] if dtype == "float32" else 0.01 + 0.01 * len(lx.CONFIGS[name]["layers"])
+
+
+def _requests(name, twice=False):
+    vocab = lx.CONFIGS[name]["vocab"]
+    req = {f"r{i}": lx.tokens(n, vocab, 100 + i) for i, n in enumerate(LENGTHS[name])}
+    if twice:
+        req.update({f"s{i}": lx.tokens(n, vocab, 200 + i)
+                    for i, n in enumerate(reversed(LENGTHS[name]))})
+    return req
+
+
+def _reference(name, requests):
+    w = None
+    out = {}
+    for rid, toks in requests.items():
+        key = (name, tuple(toks))
+        if key not in _ref:
+            w = w or lx.weights_of(name)
+            _ref[key] = P.forward(lx.CONFIGS[name], w, toks).numpy()
+        out[rid] = _ref[key]
+    return out
+
+
+def _engine(name, dtype, num_pages, poison=True, max_requests=4):
+    from zinfer_amd.engine import Engine
+    from zinfer_amd.models.build import build_model
+    store = torch.float32 if dtype == "float32" else torch.bfloat16
+    model = build_model(lx.config_of(name).model_spec(), lx.weights_of(name, dtype=store), dtype, DEV)
+    return Engine(model, page_size=lx.PAGE_SIZE[name], num_pages=num_pages,
+                  max_requests=max_requests, poison_freed=poison)
+
+
+def _replay(eng, steps):
+    from zinfer_amd.engine import StepEntry
+    outputs = {}
+    for st in steps:
+        for e in st["entries"]:
+            held = eng.length(e["id"]) if eng.has_request(e["id"]) else 0
+            assert e["start"] == held
+        logits = eng.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in st["entries"]],
+                          end=st["end"])
+        if logits.shape[0]:
+            outputs[st["step"]] = logits.cpu().numpy().copy()
+    eng.cache.check()
+    assert not eng.cache.requests
+    return outputs
+
+
+def _compare(steps, outputs, ref, vocab, dtype, name):
+    tolerance = _tol(name, dtype)
+    got = traces.collect(steps, outputs, vocab)
+    assert set(got) == set(ref)
+    worst = 0.0
+    for rid in ref:
+        assert got[rid].shape == ref[rid].shape
+        assert np.isfinite(got[rid]).all(), f"{rid}: logits are not finite"
+        err = np.abs(got[rid].astype(np.float64) - ref[rid]).max(axis=1) / np.abs(ref[rid]).max()
+        bad = np.nonzero(err > tolerance)[0]
+        assert bad.size == 0, \
+            (f"request {rid}: {bad.size} of {len(err)} positions wrong, the first {bad[0]} "
+             f"(error {err[bad[0]]:.3g} > {tolerance})")
+        worst = max(worst, float(err.max()))
+    return worst
+
+
+MODES = {"whole": traces.whole,
+         "prefill_then_single": lambda r: traces.prefill_then_single(r, tail=20),
+         "portions": traces.changing_portions, "token_by_token": traces.token_by_token,
+         "mixed": lambda r: traces.mixed(r, decode_tail=9)}
+
+
+@pytest.mark.parametrize("mode", list(MODES))
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(lx.CONFIGS))
+def test_replay_modes(name, dtype, mode):
+    requests = _requests(name, twice=mode == "mixed")
+    steps = MODES[mode](requests)
+    page = lx.PAGE_SIZE[name]
+    # the pool holds what is live at the fullest step and no more
+    pages = (traces.peak_tokens(steps, page) + page - 1) // page
+    eng = _engine(name, dtype, pages)
+    outputs = _replay(eng, steps)
+    worst = _compare(steps, outputs, _reference(name, requests), lx.CONFIGS[name]["vocab"], dtype, name)
+    if mode == "mixed":
+        assert max(len(st["entries"]) for st in steps) == 4
+        for grp in eng.cache.groups:
+            assert grp.pages.handed_out > grp.pages.num_pages, "no page was used again"
+    print(f"{name} {dtype} {mode}: error {worst:.3g}")
+
+
+@pytest.mark.parametrize("name", ["A", "C", "D"])
+def test_cut_and_batch_leave_the_bits(name):
+    """32-bit: a position's logits are the same bits whole, in portions, token by token and
+    beside other requests."""
+    requests = _requests(name)
+    vocab = lx.CONFIGS[name]["vocab"]
+    rows = []
+    for mode in ("whole", "portions", "token_by_token", "mixed"):
+        steps = MODES[mode](requests)
+        eng = _engine(name, "float32", 64, poison=False)
+        rows.append(traces.collect(steps, _replay(eng, steps), vocab))
+    for other in rows[1:]:
+        for rid in rows[0]:
+            assert np.array_equal(rows[0][rid], other[rid]), rid
+
+
+def test_pages_behind_chunks_and_windows_go_back_while_a_request_runs():
+    """A request far longer than its chunks and windows holds a few pages a layer, not its
+    length: 150 tokens run in a pool of 64."""
+    name = "A"            # chunks of 7 and 11, a window of 5, pages of 16
+    toks = lx.tokens(150, lx.CONFIGS[name]["vocab"], 7)
+    steps = traces.changing_portions({"r": toks}, sizes=(13, 2, 30, 1, 8))
+    eng = _engine(name, "float32", 4)
+    outputs = _replay(eng, steps)
+    _compare(steps, outputs, _reference(name, {"r": toks}), lx.CONFIGS[name]["vocab"], "float32", name)
+    for grp in eng.cache.groups:
+        assert grp.pages.handed_out > grp.pages.num_pages
+
+
+def test_the_residual_stream_layer_by_layer():
+    """Every layer alone (``Engine.probe_block``) on the plain implementation's stream before
+    it gives the plain implementation's stream after it, in 32-bit."""
+    name = "B"
+    toks = lx.tokens(50, lx.CONFIGS[name]["vocab"], 3)
+    streams = []
+    w = lx.weights_of(name)
+    P.forward(lx.CONFIGS[name], w, toks, streams)
+    x0 = w["embed"].double()[torch.tensor(toks)] * lx.CONFIGS[name]["embedding"]["scale"]
+    eng = _engine(name, "float32", 64, poison=False)
+    before = x0
+    for i, after in enumerate(streams):
+        got, held = eng.probe_block(i, before.to(torch.float32).to(DEV))
+        assert held == len(toks)
+        err = float((got.cpu().double() - after).abs().max() / after.abs().max())
+        assert err < 2e-5, f"layer {i}: {err:.3g}"
+        before = after
+
+
+def _write_folder(name, path, store):
+    from zinfer_amd.weights.safetensors_io import write_safetensors
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(lx.CONFIGS[name], f)
+    write_safetensors(os.path.join(path, "model.safetensors"), lx.weights_of(name, dtype=store))
+    return path
+
+
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_greedy_generation_through_entry_point_and_scheduler(name, tmp_path):
+    """Prompts of unequal length generate together; every request's tokens are the plain
+    implementation's arg-max wherever that one is clear."""
+    from zinfer_amd.entrypoints import LLM, SamplingParams
+    path = _write_folder(name, str(tmp_path / name), torch.float32)
+    vocab = lx.CONFIGS[name]["vocab"]
+    prompts = [lx.tokens(n, vocab, 300 + n) for n in (3, 41, 18, 7, 29)]
+    llm = LLM(path, dtype="float32", device=DEV, page_size=lx.PAGE_SIZE[name], max_tokens=512,
+              max_step_tokens=48, chunk_size=16, max_seqs=4)
+    n_new = 14
+    outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=n_new,
+                                                ignore_eos=True))
+    w = lx.weights_of(name)
+    for prompt, got in zip(prompts, outs):
+        assert len(got) == n_new
+        logits = P.forward(lx.CONFIGS[name], w, list(prompt) + list(got))
+        for i, tok in enumerate(got):
+            row = logits[len(prompt) - 1 + i]
+            top2 = torch.topk(row, 2).values
+            if float(top2[0] - top2[1]) > 1e-3 * float(row.abs().max()):
+                assert int(row.argmax()) == tok, f"token {i} of a prompt of {len(prompt)}"
+
+
+def test_long_generation_in_bfloat16_stays_finite_and_uses_graphs(tmp_path):
+    """Sixty tokens decoded behind a prompt, many times the windows and chunks, through the
+    scheduler's runs of decode steps: the steps replay as graphs and the tokens are ids."""
+    from zinfer_amd.entrypoints import LLM, SamplingParams
+    name = "D"
+    path = _write_folder(name, str(tmp_path / name), torch.bfloat16)
+    llm = LLM(path, dtype="bfloat16", device=DEV, page_size=16, max_tokens=512, max_seqs=4)
+    prompts = [lx.tokens(n, 512, 400 + n) for n in (5, 70)]
+    outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=60, ignore_eos=True))
+    assert all(len(o) == 60 and all(0 <= t < 512 for t in o) for o in outs)
+    assert llm.engine.graph_replays > 0
+
+
+def test_replay_program_on_a_model_folder(tmp_path):
+    """``bin/trace_run`` chooses the model class by config.json and writes the logits of a
+    mixed trace; both dtypes."""
+    name = "A"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    requests = _requests(name)
+    steps = traces.mixed(requests, decode_tail=5)
+    text = "".join(json.dumps({k: v for k, v in st.items()}) + "\n" for st in steps)
+    ref = _reference(name, requests)
+    for dtype in ("float32", "bfloat16"):
+        store = torch.float32 if dtype == "float32" else torch.bfloat16
+        path = _write_folder(name, str(tmp_path / dtype), store)
+        out = str(tmp_path / ("out_" + dtype))
+        r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", path,
+                            "--dtype", dtype, "--out", out, "--max-tokens",
+                            str(traces.peak_tokens(steps, 64))],
+                           input=text, capture_output=True, text=True, timeout=300)
+        assert r.returncode == 0, r.stderr[-2000:]
+        done = [l for l in r.stdout.splitlines() if l.startswith("done ")]
+        assert done == [f"done {st['step']}" for st in steps]
+        outputs = {st["step"]: np.fromfile(os.path.join(out, f"{st['step']}.f32"), dtype="<f4")
+                   for st in steps if any(e["want"] for e in st["entries"])}
+        _compare(steps, outputs, ref, lx.CONFIGS[name]["vocab"], dtype, name)
+
+
+def test_generation_through_the_command_line(tmp_path):
+    """``bin/zinfer generate-token-ids`` on a Lodenex folder: the oracle's greedy tokens."""
+    name = "A"
+    path = _write_folder(name, str(tmp_path / name), torch.float32)
+    prompt = lx.tokens(11, lx.CONFIGS[name]["vocab"], 9)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "zinfer"), "generate-token-ids",
+                        path, ",".join(map(str, prompt)), "6", "--dtype", "float32"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    line = [l for l in r.stdout.splitlines() if l.startswith("tokens: ")][0]
+    got = json.loads(line[len("tokens: "):])
+    assert got[:len(prompt)] == prompt and len(got) == len(prompt) + 6
+    w = lx.weights_of(name)
+    logits = P.forward(lx.CONFIGS[name], w, got[:-1])
+    for i in range(len(prompt) - 1, len(got) - 1):
+        top2 = torch.topk(logits[i], 2).values
+        if float(top2[0] - top2[1]) > 1e-3 * float(logits[i].abs().max()):
+            assert int(logits[i].argmax()) == got[i + 1]
