@@ -156,6 +156,7 @@ TESTED_AGAINST = {
     "activation": "plain_lodenex.py:gelu_erf", "norm_add_store": "plain_lodenex.py:rms_norm",
     "project_rows": "plain_lodenex.py:rotate_leading",
     "masked_attention": "plain_lodenex.py:masked_softmax_values",
+    "masked_attention_mfma": "plain_lodenex.py:masked_softmax_values",
     "head_products": "test_lodenex_kernels_gpu.py:test_head_products",
 }
 

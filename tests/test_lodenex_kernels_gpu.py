@@ -353,3 +353,126 @@ def test_pages_before_the_mask_are_not_touched():
         assert first > 2
         pg.table[0, :first] = -1
         assert torch.equal(_run(pg, [q], [5], torch.float32, H, 0.4, 0.0, window, chunk), full)
+
+
+# ------------------------------------------------------------------------------ the MFMA form
+def _run_mfma(pg, qs, q_lens, H, scale, cap=0.0, window=0, chunk=0, sink=None, gate=None,
+              gate_mode=None, tied=None, n_splits=None):
+    dt = torch.bfloat16
+    T = sum(q_lens)
+    q = torch.cat(qs).reshape(T, -1).to(DEV)
+    VW = tied if tied else pg.VW
+    out = torch.zeros((T, H * VW), dtype=dt, device=DEV)
+    q_start = [0]
+    for n in q_lens:
+        q_start.append(q_start[-1] + n)
+    ops.masked_attention_mfma(q, None if gate is None else gate.to(DEV), gate_mode, pg.k_pool,
+                              None if tied else pg.v_pool, None if sink is None else sink.to(DEV),
+                              pg.table, _i32(q_start), _i32(pg.lens), out, scale, cap, window,
+                              chunk, H, pg.G, pg.KW, VW, pg.ps, max(q_lens), max(pg.lens),
+                              n_splits=n_splits)
+    return out
+
+
+MFMA_CASES = [  # H, G, KW, VW, tied, page, lens, q_lens, cap, window, chunk
+    (4, 2, 96, 96, False, 16, [230, 90, 33], [230, 90, 33], 20.0, 0, 120),
+    (8, 8, 64, 64, False, 16, [300, 41], [77, 2], 0.0, 100, 0),
+    (32, 1, 128, 128, False, 16, [150], [150], 5.0, 0, 1000),
+    (6, 1, 160, 128, True, 16, [200, 64], [200, 10], 0.0, 40, 0),
+    (3, 1, 96, 64, True, 8, [333], [333], 0.0, 0, 0),
+    (16, 1, 192, 128, True, 16, [500], [100], 0.0, 256, 0),
+    (12, 4, 128, 128, False, 32, [700], [700], 30.0, 0, 0),
+]
+
+
+@pytest.mark.parametrize("case", MFMA_CASES)
+def test_mfma_attention_against_plain(case):
+    H, G, KW, VW, tied, ps, lens, q_lens, cap, window, chunk = case
+    dt = torch.bfloat16
+    pg = Paged(lens, G, KW, 0 if tied else VW, ps, dt, 3)
+    scale = 1.3 / math.sqrt(KW)
+    sink = None if tied else _rand((H,), 5, 1.5)
+    T = sum(q_lens)
+    qs = [_rand((n, H, KW), 20 + i, 1.0, dt) for i, n in enumerate(q_lens)]
+    gate = _rand((T, H * VW), 7, 1.5, dt) if tied else _rand((T, H), 6, 1.5, dt)
+    mode = "element" if tied else "head"
+    vals = [k[..., :VW] for k in pg.k] if tied else pg.v
+    want = torch.cat([_plain_attention(q, pg.k[s], vals[s], H, G, scale, cap, window, chunk, sink)
+                      for s, q in enumerate(qs)])
+    g64 = torch.sigmoid(gate.double())
+    want_g = want * (g64.view(T, H, VW) if tied else g64[:, :, None])
+    assert ops.masked_attention_mfma_covers(dt, H, G, KW, VW, tied)
+    for parts in (None, 1, 2, 4):
+        out = _run_mfma(pg, qs, q_lens, H, scale, cap, window, chunk, sink, gate, mode,
+                        tied=VW if tied else None, n_splits=parts)
+        assert rel_err(out.view(T, H, VW), want_g) < 2 * tol(dt), parts
+    # the 32-bit kernel on the same operands agrees
+    ref = _run(pg, qs, q_lens, dt, H, scale, cap, window, chunk, sink, gate, mode,
+               tied=VW if tied else None)
+    assert rel_err(out, ref.double()) < 2 * tol(dt)
+
+
+@pytest.mark.parametrize("case", MFMA_CASES)
+def test_mfma_decode_steps_against_plain(case):
+    """One token a sequence, the contexts split over 1, 2 and 5 workgroups of four waves."""
+    H, G, KW, VW, tied, ps, lens, _, cap, window, chunk = case
+    dt = torch.bfloat16
+    lens = lens + [1, 31, 32, 33]
+    pg = Paged(lens, G, KW, 0 if tied else VW, ps, dt, 4)
+    scale = 1.1 / math.sqrt(KW)
+    sink = None if tied else _rand((H,), 5, 1.5)
+    n = len(lens)
+    qs = [_rand((1, H, KW), 60 + i, 1.0, dt) for i in range(n)]
+    gate = _rand((n, H * VW), 7, 1.5, dt) if tied else _rand((n, H), 6, 1.5, dt)
+    mode = "element" if tied else "head"
+    vals = [k[..., :VW] for k in pg.k] if tied else pg.v
+    want = torch.cat([_plain_attention(q, pg.k[s], vals[s], H, G, scale, cap, window, chunk, sink)
+                      for s, q in enumerate(qs)])
+    g64 = torch.sigmoid(gate.double())
+    want_g = want * (g64.view(n, H, VW) if tied else g64[:, :, None])
+    for blocks in (None, 1, 2, 5):
+        out = _run_mfma(pg, qs, [1] * n, H, scale, cap, window, chunk, sink, gate, mode,
+                        tied=VW if tied else None, n_splits=blocks)
+        assert rel_err(out.view(n, H, VW), want_g) < 2 * tol(dt), blocks
+
+
+@pytest.mark.parametrize("decode", [False, True])
+def test_mfma_a_loud_key_at_the_edges(decode):
+    dt = torch.bfloat16
+    H, G, KW, VW, ps, n = 2, 1, 64, 64, 16, 333
+    qv = torch.zeros((H, KW))
+    qv[:, 0] = 1.0
+    T = 1 if decode else 37
+    for name, at, window, chunk, seen in (("far", 3, 0, 0, True), ("first", 0, 0, 0, True),
+                                          ("window_in", n - 50, 50, 0, True),
+                                          ("window_out", n - 51, 50, 0, False),
+                                          ("chunk_in", 320, 0, 64, True),
+                                          ("chunk_out", 319, 0, 64, False),
+                                          ("page_border", 320, 13, 0, True),
+                                          ("split_border", 256, 0, 0, True)):
+        k, v = _planted(n, G, KW, VW, at, dt, 40)
+        pg = Paged([n], G, KW, VW, ps, dt, 11, k=[k], v=[v])
+        q = qv.to(dt).expand(T, H, KW).contiguous()
+        for splits in (None, 3):
+            out = _run_mfma(pg, [q], [T], H, 1.0, 0.0, window, chunk, n_splits=splits)
+            last = out.view(T, H, VW)[-1].float().cpu()
+            if seen:
+                assert float((last - 5.0).abs().max()) < 0.05, name
+            else:
+                assert float(last.abs().max()) < 1.5, name
+            want = _plain_attention(q, k, v, H, G, 1.0, 0.0, window, chunk, None)
+            assert rel_err(out.view(T, H, VW), want) < 2 * tol(dt), name
+
+
+def test_mfma_pages_before_the_mask_are_not_touched():
+    H, G, KW, VW, ps, n = 4, 2, 64, 64, 16, 301
+    dt = torch.bfloat16
+    for window, chunk in ((40, 0), (0, 64)):
+        for T in (1, 45):
+            pg = Paged([n], G, KW, VW, ps, dt, 13)
+            q = _rand((T, H, KW), 1, 1.0, dt)
+            full = _run_mfma(pg, [q], [T], H, 0.2, 0.0, window, chunk)
+            first = (n - T - window + 1 if window else (n - T) // chunk * chunk) // ps
+            assert first > 2
+            pg.table[0, :first] = -1
+            assert torch.equal(_run_mfma(pg, [q], [T], H, 0.2, 0.0, window, chunk), full)

@@ -401,3 +401,418 @@ extern "C" int zf_head_products(const void* a, int dtype, long long a_stride, in
 #undef HP_LAUNCH
   ZF_CHECK_LAUNCH();
 }
+
+// =====================================================================================
+//  bfloat16 MFMA kernels: waves on their own
+// =====================================================================================
+// The same attention in v_mfma_f32_32x32x16_bf16 tiles, for key rows of KD and value rows of VD
+// elements (KD a multiple of 16, VD of 32) and at most 32 query heads a kv head.  A wave takes
+// 32 rows, (position, head of the group) pairs of one sequence, and walks the keys those rows
+// see in chunks of 32, on its own: no barrier between waves anywhere.  A lane loads, for its
+// key of the chunk, the 8 values that its operand of S^T = K Q^T needs straight from the pool
+// (every value of the chunk once in the wave), and the 8 values of that key's value row
+// (TIED: of the key row's leading columns) that it writes transposed (permuted against bank
+// conflicts) into the wave's own LDS tile for O^T = V^T P^T.  The score tile is transposed so
+// that a lane's 16 scores belong to one row: cap, mask and soft-max run in registers in 32-bit
+// (base-2 exponentials, the scale folded in; with a sink the running maximum starts at the
+// sink and the sum at 1).  Each weight enters the second product as the sum of two bfloat16
+// numbers (its rounding and the rounding of what that leaves).  The next chunk's keys are asked
+// for as soon as this chunk's score products are issued, its values once this chunk's are in
+// the tile.
+//   DECODE: grid (sequence, kv head, block); one token a sequence, its G heads the first G rows;
+//   the four waves of a workgroup are four splits of the context, wave_keys keys each.
+//   else: grid (tile of 128 / G positions, kv head, part); with several parts a wave takes that
+//   part of its keys.  Splits and parts leave un-normalised partials (maximum, sum, O) that
+//   masked_attention_merge_kernel combines in split order; the sink belongs to the first.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 mw_bf16x8_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float mw_f32x16_t;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t mw_u32x4_t;
+
+#define MW_ROWS 128
+#define MW_KEYS 32
+#define MW_LOG2E 1.4426950408889634f
+
+__device__ __forceinline__ float mw_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+// where key j of value element d lies in the [d][key] tile
+__device__ __forceinline__ int mw_swz(int j, int d) { return (((j >> 2) ^ ((d >> 3) & 7)) << 2) | (j & 3); }
+// tanh through one exponential: 1 - 2 / (e^(2x) + 1); +-1 where the exponential leaves the range
+__device__ __forceinline__ float mw_tanh(float x) {
+  const float e = mw_exp2(x * (2.0f * MW_LOG2E));
+  return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+}
+
+struct MaskedWaveArgs {
+  long long q_stride, gate_stride;
+  float scale, cap;
+  int window, chunk, gate_mode;
+  int n_seqs, nH, nKV, page_size, max_pages, QT, wave_keys;
+};
+
+template <int KD, int VD, bool TIED, bool DECODE>
+__global__ __launch_bounds__(256, 2) void masked_attention_wave_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ gate,
+    const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
+    const float* __restrict__ sink, const int* __restrict__ block_table,
+    const int* __restrict__ q_start, const int* __restrict__ ctx_len, bf16_t* __restrict__ out,
+    float* __restrict__ ws_o, float* __restrict__ ws_ml, MaskedWaveArgs a) {
+  constexpr int LDT = MW_KEYS + 4;
+  __shared__ __attribute__((aligned(16))) bf16_t vt_all[4 * VD * LDT];
+  const int kvh = blockIdx.y;
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int c = lane % 32, hl = lane / 32;
+  bf16_t* vt = vt_all + wave * VD * LDT;
+  const int G = a.nH / a.nKV;
+  const int window = a.window, chunk = a.chunk, page_size = a.page_size, nKV = a.nKV;
+
+  // the first key position p sees
+  auto first_seen = [&](int p) {
+    int lo = 0;
+    if (window > 0 && p - window + 1 > lo) lo = p - window + 1;
+    if (chunk > 0 && p / chunk * chunk > lo) lo = p / chunk * chunk;
+    return lo;
+  };
+
+  int s, tok, pos_r, lo_r, h, split = 0, n_splits = 1;
+  int k_first, k_end;          // the keys the wave walks: [k_first down to a multiple of 32, k_end)
+  bool row_ok;
+  if constexpr (DECODE) {
+    s = blockIdx.x;
+    split = blockIdx.z * 4 + wave;
+    n_splits = gridDim.z * 4;
+    row_ok = c < G;
+    h = kvh * G + (row_ok ? c : 0);
+    tok = s;
+    pos_r = ctx_len[s] - 1;
+    lo_r = first_seen(pos_r);
+    k_first = lo_r;
+    k_end = pos_r + 1;
+  } else {
+    split = blockIdx.z;
+    n_splits = gridDim.z;
+    s = 0;
+    int tile = blockIdx.x;
+    for (; s < a.n_seqs; ++s) {
+      const int n = (q_start[s + 1] - q_start[s] + a.QT - 1) / a.QT;
+      if (tile < n) break;
+      tile -= n;
+    }
+    if (s >= a.n_seqs) return;
+    const int q_len = q_start[s + 1] - q_start[s];
+    const int first = tile * a.QT;
+    const int npos = min(a.QT, q_len - first);
+    const int nrows = npos * G;
+    if (wave * 32 >= nrows) return;                // (no barrier follows: waves are on their own)
+    const int pos0 = ctx_len[s] - q_len + first;
+    const int row = wave * 32 + c;
+    row_ok = row < nrows;
+    const int qi = row_ok ? row / G : 0;
+    h = kvh * G + (row_ok ? row % G : 0);
+    tok = q_start[s] + first + qi;
+    pos_r = pos0 + qi;
+    lo_r = first_seen(pos_r);
+    const int p_lo = pos0 + (wave * 32) / G;                       // the wave's first position
+    const int p_hi = pos0 + (min(nrows, wave * 32 + 32) - 1) / G;  // and its last
+    k_first = first_seen(p_lo);        // (the first key a position sees never moves back)
+    k_end = p_hi + 1;
+  }
+  const int* table = block_table + (size_t)s * a.max_pages;
+
+  mw_bf16x8_t qf[KD / 16];
+  {
+    const bf16_t* qrow = q + (size_t)tok * a.q_stride + (size_t)h * KD;
+#pragma unroll
+    for (int i = 0; i < KD / 16; ++i) {
+      mw_u32x4_t v = {0u, 0u, 0u, 0u};
+      if (row_ok) v = *(const mw_u32x4_t*)(qrow + 16 * i + 8 * hl);
+      qf[i] = *(const mw_bf16x8_t*)&v;
+    }
+  }
+  mw_f32x16_t acc[VD / 32];
+#pragma unroll
+  for (int i = 0; i < VD / 32; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
+  // scores are kept times log2(e), so that every weight is one v_exp_f32
+  const float scale_log2 = a.scale * MW_LOG2E;
+  const float cap_log2 = a.cap * MW_LOG2E;
+  const float inv_cap = a.cap > 0.f ? a.scale / a.cap : 0.f;
+  const bool capped = a.cap > 0.f;
+  const bool has_sink = sink != nullptr && split == 0;
+  float m = -INFINITY, l = 0.f;
+  if (has_sink) {
+    m = sink[h] * MW_LOG2E;
+    l = 1.f;
+  }
+
+  int k_begin = k_first / MW_KEYS * MW_KEYS;
+  if constexpr (DECODE) {
+    k_begin += split * a.wave_keys;
+    k_end = min(k_end, k_begin + a.wave_keys);
+  } else if (n_splits > 1) {
+    const int share = (k_end - k_begin + n_splits * MW_KEYS - 1) / (n_splits * MW_KEYS) * MW_KEYS;
+    k_begin += split * share;
+    k_end = min(k_end, k_begin + share);
+  }
+
+  // this lane's key of a chunk: key base + c; of its key row the values 16 i + 8 hl .. + 8 for
+  // every i, of its value row the same
+  mw_u32x4_t kf[KD / 16];
+  mw_u32x4_t vf[TIED ? 1 : VD / 16];
+  auto row_of = [&](int base, bool& ok) {
+    const int key = base + c;
+    ok = key >= k_first && key < k_end;          // (pages before k_first may have gone back)
+    size_t prow = 0;
+    if (ok) prow = ((size_t)table[key / page_size] * nKV + kvh) * page_size + key % page_size;
+    return prow;
+  };
+  auto fetch_k = [&](int base) {
+    bool ok;
+    const size_t prow = row_of(base, ok);
+#pragma unroll
+    for (int i = 0; i < KD / 16; ++i) {
+      mw_u32x4_t v = {0u, 0u, 0u, 0u};
+      if (ok) v = *(const mw_u32x4_t*)(k_pool + prow * KD + 16 * i + 8 * hl);
+      kf[i] = v;
+    }
+  };
+  auto fetch_v = [&](int base) {
+    if constexpr (!TIED) {
+      bool ok;
+      const size_t prow = row_of(base, ok);
+#pragma unroll
+      for (int i = 0; i < VD / 16; ++i) {
+        mw_u32x4_t v = {0u, 0u, 0u, 0u};
+        if (ok) v = *(const mw_u32x4_t*)(v_pool + prow * VD + 16 * i + 8 * hl);
+        vf[i] = v;
+      }
+    }
+  };
+  if (k_begin < k_end) {
+    fetch_k(k_begin);
+    fetch_v(k_begin);
+  }
+  for (int base = k_begin; base < k_end; base += MW_KEYS) {
+    const bool more = base + MW_KEYS < k_end;
+    mw_f32x16_t sc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+#pragma unroll
+    for (int i = 0; i < KD / 16; ++i)
+      sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const mw_bf16x8_t*)&kf[i], qf[i], sc, 0, 0, 0);
+    // the chunk's values transposed into the wave's tile
+#pragma unroll
+    for (int i = 0; i < VD / 16; ++i) {
+      const bf16_t* e = TIED ? (const bf16_t*)&kf[i] : (const bf16_t*)&vf[TIED ? 0 : i];
+#pragma unroll
+      for (int x = 0; x < 8; ++x)
+        vt[(16 * i + 8 * hl + x) * LDT + mw_swz(c, 16 * i + 8 * hl)] = e[x];
+    }
+    if (more) {                                     // in flight while this chunk runs
+      fetch_k(base + MW_KEYS);
+      fetch_v(base + MW_KEYS);
+    }
+    float cmax = -INFINITY;
+    if (capped) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sc[r] = cap_log2 * mw_tanh(sc[r] * inv_cap);
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sc[r] *= scale_log2;
+    }
+    // a chunk that every row of the wave sees whole needs no mask
+    const bool whole = row_ok && base >= lo_r && base + MW_KEYS - 1 <= pos_r &&
+                       base >= k_first && base + MW_KEYS <= k_end;
+    if (__all(whole)) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) cmax = fmaxf(cmax, sc[r]);
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = base + 8 * (r / 4) + 4 * hl + r % 4;
+        const bool seen = row_ok && key >= lo_r && key <= pos_r && key >= k_first && key < k_end;
+        sc[r] = seen ? sc[r] : -INFINITY;
+        cmax = fmaxf(cmax, sc[r]);
+      }
+    }
+    cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));
+    const float m_new = fmaxf(m, cmax);
+    // nothing seen yet (and no sink): every weight below is exp(-inf) = 0
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float corr = mw_exp2(m - m_use);
+    float psum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      sc[r] = mw_exp2(sc[r] - m_use);
+      psum += sc[r];
+    }
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * corr + psum;
+    m = m_new;
+    if (__any(corr != 1.0f)) {                     // (the maximum of some row moved)
+#pragma unroll
+      for (int i = 0; i < VD / 32; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][r] *= corr;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();               // the wave's transposed tile is written
+    // O^T += V^T P^T over the chunk's two groups of 16 keys; the registers 8 t .. 8 t + 7 hold
+    // the weights of the keys 16 t + {0..3, 8..11} + 4 hl, and V^T is read in that same order
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      mw_bf16x8_t p_hi, p_lo;
+#pragma unroll
+      for (int x = 0; x < 8; ++x) {
+        const float p = sc[8 * t + x];
+        const __bf16 hi = (__bf16)p;
+        p_hi[x] = hi;
+        p_lo[x] = (__bf16)(p - (float)hi);
+      }
+#pragma unroll
+      for (int i = 0; i < VD / 32; ++i) {
+        const bf16_t* src = vt + (i * 32 + c) * LDT;
+        const uint2 a0 = *(const uint2*)(src + mw_swz(16 * t + 4 * hl, i * 32 + c));
+        const uint2 a1 = *(const uint2*)(src + mw_swz(16 * t + 8 + 4 * hl, i * 32 + c));
+        mw_u32x4_t av = {a0.x, a0.y, a1.x, a1.y};
+        const mw_bf16x8_t vv = *(const mw_bf16x8_t*)&av;
+        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vv, p_hi, acc[i], 0, 0, 0);
+        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vv, p_lo, acc[i], 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    __builtin_amdgcn_wave_barrier();               // the tile is read before it is written again
+  }
+  if (!row_ok) return;
+  // acc[i][r] is element d = 32 i + 8 (r / 4) + 4 hl + r % 4 of this lane's row
+  if (DECODE || n_splits > 1) {
+    const size_t slot = ((size_t)tok * a.nH + h) * n_splits + split;
+    float* po = ws_o + slot * VD;
+#pragma unroll
+    for (int i = 0; i < VD / 32; ++i)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4)
+        *(float4*)(po + 32 * i + 8 * r4 + 4 * hl) = make_float4(acc[i][4 * r4], acc[i][4 * r4 + 1],
+                                                                acc[i][4 * r4 + 2], acc[i][4 * r4 + 3]);
+    if (hl == 0) {
+      ws_ml[2 * slot] = m;
+      ws_ml[2 * slot + 1] = l;
+    }
+  } else {
+    float inv = 1.0f / l;
+    if (a.gate_mode == MA_GATE_HEAD)
+      inv *= 1.0f / (1.0f + expf(-bf16_to_float(gate[(size_t)tok * a.gate_stride + h])));
+    bf16_t* orow = out + ((size_t)tok * a.nH + h) * VD;
+    const bf16_t* grow = a.gate_mode == MA_GATE_ELEMENT
+        ? gate + (size_t)tok * a.gate_stride + (size_t)h * VD : nullptr;
+#pragma unroll
+    for (int i = 0; i < VD / 32; ++i)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const int d = 32 * i + 8 * r4 + 4 * hl;
+        float v[4];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+          v[x] = acc[i][4 * r4 + x] * inv;
+          if (grow != nullptr) v[x] *= 1.0f / (1.0f + expf(-bf16_to_float(grow[d + x])));
+        }
+        *(uint2*)(orow + d) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+      }
+  }
+}
+
+// one wave per (token, head): the splits' partials in split order (their maxima are scores
+// times log2(e)), then the gate
+__global__ __launch_bounds__(ZF_WAVE) void masked_attention_merge_kernel(
+    const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
+    const bf16_t* __restrict__ gate, long long gate_stride, int gate_mode,
+    bf16_t* __restrict__ out, int nH, int vd, int n_splits) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const size_t slot0 = ((size_t)t * nH + h) * n_splits;
+  // lane z holds split z's maximum and sum (at most 64 splits); a split without keys has the
+  // maximum -inf and counts for nothing
+  float mz = -INFINITY, lz = 0.f;
+  if (lane < n_splits) {
+    mz = ws_ml[2 * (slot0 + lane)];
+    lz = ws_ml[2 * (slot0 + lane) + 1];
+  }
+  const float M = wave_max(mz);
+  __shared__ float w[ZF_WAVE], lw[ZF_WAVE];
+  w[lane] = mz == -INFINITY ? 0.f : exp2f(mz - M);
+  lw[lane] = lz * w[lane];
+  __syncthreads();
+  float L = 0.f;
+  for (int z = 0; z < n_splits; ++z) L += lw[z];
+  float inv = 1.0f / L;
+  if (gate_mode == MA_GATE_HEAD)
+    inv *= 1.0f / (1.0f + expf(-bf16_to_float(gate[(size_t)t * gate_stride + h])));
+  for (int d = lane; d < vd; d += ZF_WAVE) {
+    float o = 0.f;
+    for (int z = 0; z < n_splits; ++z) o += ws_o[(slot0 + z) * vd + d] * w[z];
+    o *= inv;
+    if (gate_mode == MA_GATE_ELEMENT)
+      o *= 1.0f / (1.0f + expf(-bf16_to_float(gate[(size_t)t * gate_stride + (size_t)h * vd + d])));
+    out[((size_t)t * nH + h) * vd + d] = float_to_bf16(o);
+  }
+}
+
+#define MW_LAUNCH(KD, VD, TIED, DEC)                                                             \
+  hipLaunchKernelGGL((masked_attention_wave_kernel<KD, VD, TIED, DEC>), grid, dim3(256), 0,      \
+                     stream, (const bf16_t*)q, (const bf16_t*)gate, (const bf16_t*)k_pool,       \
+                     (const bf16_t*)v_pool, sink, block_table, q_start, ctx_len, (bf16_t*)out,   \
+                     ws_o, ws_ml, a)
+
+// the shapes that are built: values of their own as wide as the keys; and the keys' leading
+// columns as values (a latent and a rotated part behind it)
+#define MW_SHAPES(DEC)                                                                           \
+  if (!tied && KD == 64 && VD == 64) MW_LAUNCH(64, 64, false, DEC);                              \
+  else if (!tied && KD == 96 && VD == 96) MW_LAUNCH(96, 96, false, DEC);                         \
+  else if (!tied && KD == 128 && VD == 128) MW_LAUNCH(128, 128, false, DEC);                     \
+  else if (tied && KD == 96 && VD == 64) MW_LAUNCH(96, 64, true, DEC);                           \
+  else if (tied && KD == 160 && VD == 128) MW_LAUNCH(160, 128, true, DEC);                       \
+  else if (tied && KD == 192 && VD == 128) MW_LAUNCH(192, 128, true, DEC);                       \
+  else return -3
+
+// decode == 0: a step's tokens in tiles of 128 / G positions, n_tiles an upper bound of the
+// tiles over all sequences (workgroups beyond the real number leave at once), every wave's keys
+// in n_splits parts.  decode != 0: token s is sequence s's one token; n_splits workgroups a
+// (sequence, kv head), every wave a split of wave_keys keys (a multiple of 32).  With partial
+// results: ws_o [T * nH * splits * VD], ws_ml [T * nH * splits * 2] floats, splits = n_splits
+// (decode: 4 n_splits), at most 64.
+extern "C" int zf_masked_attention_mfma(const void* q, long long q_stride, const void* gate,
+                                        long long gate_stride, int gate_mode, const void* k_pool,
+                                        const void* v_pool, const float* sink,
+                                        const int* block_table, const int* q_start,
+                                        const int* ctx_len, void* out, float* ws_o, float* ws_ml,
+                                        float scale, float cap, int window, int chunk, int T,
+                                        int n_seqs, int n_tiles, int nH, int nKV, int KD, int VD,
+                                        int page_size, int max_pages, int decode, int n_splits,
+                                        int wave_keys, hipStream_t stream) {
+  if (T <= 0) return 0;
+  const int splits = decode ? 4 * n_splits : n_splits;
+  if (nKV <= 0 || nH % nKV != 0 || nH / nKV > 32 || page_size <= 0 || n_splits < 1 ||
+      splits > ZF_WAVE || ((decode || n_splits > 1) && (!ws_o || !ws_ml)) ||
+      (decode && (wave_keys <= 0 || wave_keys % MW_KEYS != 0 || T != n_seqs)) ||
+      gate_mode < 0 || gate_mode > 2 || (gate_mode != MA_GATE_NONE && gate == nullptr) ||
+      window < 0 || chunk < 0 || cap < 0.f)
+    return -2;
+  const bool tied = v_pool == nullptr;
+  MaskedWaveArgs a;
+  a.q_stride = q_stride; a.gate_stride = gate_stride; a.scale = scale; a.cap = cap;
+  a.window = window; a.chunk = chunk; a.gate_mode = gate_mode; a.n_seqs = n_seqs; a.nH = nH;
+  a.nKV = nKV; a.page_size = page_size; a.max_pages = max_pages;
+  a.QT = decode ? 1 : MW_ROWS / (nH / nKV);
+  a.wave_keys = wave_keys;
+  if (decode) {
+    dim3 grid(n_seqs, nKV, n_splits);
+    MW_SHAPES(true);
+  } else {
+    if (n_tiles <= 0) return 0;
+    dim3 grid(n_tiles, nKV, n_splits);
+    MW_SHAPES(false);
+  }
+  if (decode || n_splits > 1)
+    hipLaunchKernelGGL(masked_attention_merge_kernel, dim3(T, nH), dim3(ZF_WAVE), 0, stream, ws_o,
+                       ws_ml, (const bf16_t*)gate, gate_stride, gate_mode, (bf16_t*)out, nH, VD,
+                       splits);
+  ZF_CHECK_LAUNCH();
+}

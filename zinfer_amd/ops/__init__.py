@@ -2032,7 +2032,8 @@ def _masked_attention_checks(what, q, gate, gate_mode, k_pool, v_pool, sink, blo
                                 "the sink float32 [nH]")
     for t, name in ((block_table, "block_table"), (q_start, "q_start"), (ctx_len, "ctx_len"),
                     (seq_index, "seq_index")):
-        _i32(t, name)
+        if t is not None:
+            _i32(t, name)
     if n_kv_heads <= 0 or n_heads % n_kv_heads != 0:
         raise KernelUnavailable(f"{what}: InvalidGrouping")
     if key_width < 1 or not 0 < value_width <= MAX_HEAD_DIM \
@@ -2043,7 +2044,8 @@ def _masked_attention_checks(what, q, gate, gate_mode, k_pool, v_pool, sink, blo
         raise KernelUnavailable(f"{what}: block table shorter than the context")
     n_seqs = ctx_len.shape[0]
     if q_start.shape[0] != n_seqs + 1 or block_table.shape[0] != n_seqs \
-            or seq_index.shape[0] != T or not block_table.is_contiguous() \
+            or (seq_index is not None and seq_index.shape[0] != T) \
+            or not block_table.is_contiguous() \
             or not k_pool.is_contiguous() or (v_pool is not None and not v_pool.is_contiguous()):
         raise KernelUnavailable(f"{what}: per-sequence arrays disagree in length")
 
@@ -2111,3 +2113,105 @@ def head_products(a: torch.Tensor, a_off: int, a_hd: int, w: torch.Tensor,
         _ptr(a), _dt(a), ctypes.c_longlong(a_stride), int(a_off), int(a_hd), _ptr(w), _dt(w),
         _ptr(gate), ctypes.c_longlong(g_stride), _ptr(out), ctypes.c_longlong(o_stride),
         int(out_off), int(out_hd), T, H, N, K, _stream()), "head_products")
+
+
+# (key width, value width) the MFMA kernels are built for: values of their own, and the keys'
+# leading columns as values
+MASKED_MFMA_SHAPES = {False: ((64, 64), (96, 96), (128, 128)),
+                      True: ((96, 64), (160, 128), (192, 128))}
+MASKED_MFMA_ROWS = 128           # (position, head) pairs a workgroup takes
+MASKED_ROWS_WAVES = 2048         # a prompt portion's keys are cut in parts until this many waves run
+MASKED_ROWS_MAX_PARTS = 4
+MASKED_DECODE_WORKGROUPS = 1024  # a decode step's contexts are split until about this many run
+
+
+def masked_attention_mfma_covers(dtype, n_heads: int, n_kv_heads: int, key_width: int,
+                                 value_width: int, tied: bool) -> bool:
+    """Whether the bfloat16 MFMA kernels take the shape; otherwise (and in 32-bit) the kernel
+    for every size runs."""
+    return dtype == torch.bfloat16 and (key_width, value_width) in MASKED_MFMA_SHAPES[bool(tied)] \
+        and n_heads // n_kv_heads <= 32
+
+
+def attend_masked(q, gate, gate_mode, k_pool, v_pool, sink, block_table, q_start, ctx_len,
+                  seq_index, out, scale, cap, window, chunk, n_heads, n_kv_heads, key_width,
+                  value_width, page_size, max_q_len, max_ctx_len) -> None:
+    """``masked_attention`` through the fastest kernel that takes the shape: in bfloat16, for
+    the widths of ``MASKED_MFMA_SHAPES``, the MFMA kernels (``masked_attention_mfma``); else
+    the 32-bit kernel.  Same arguments, same result up to rounding."""
+    if masked_attention_mfma_covers(q.dtype, n_heads, n_kv_heads, key_width, value_width,
+                                    v_pool is None) \
+            and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0:
+        masked_attention_mfma(q, gate, gate_mode, k_pool, v_pool, sink, block_table, q_start,
+                              ctx_len, out, scale, cap, window, chunk, n_heads, n_kv_heads,
+                              key_width, value_width, page_size, max_q_len, max_ctx_len)
+    else:
+        masked_attention(q, gate, gate_mode, k_pool, v_pool, sink, block_table, q_start, ctx_len,
+                         seq_index, out, scale, cap, window, chunk, n_heads, n_kv_heads,
+                         key_width, value_width, page_size, max_ctx_len)
+
+
+@_launches("attention")
+def masked_attention_mfma(q, gate, gate_mode, k_pool, v_pool, sink, block_table, q_start, ctx_len,
+                          out, scale, cap, window, chunk, n_heads, n_kv_heads, key_width,
+                          value_width, page_size, max_q_len, max_ctx_len,
+                          n_splits: Optional[int] = None) -> None:
+    """The bfloat16 MFMA form of ``masked_attention`` (see there for the arguments).  Scores, cap
+    and soft-max are 32-bit; a weight enters the second product as the sum of two bfloat16
+    numbers.  Every wave takes 32 (position, head) rows and walks their keys on its own.  A step
+    in which every sequence brings one token runs the decode form: each context is split over
+    ``n_splits`` workgroups of four waves that are splits of their own (None: by the block
+    table's width and the window or chunk, never by the contexts themselves, so that a captured
+    step replays for other contexts) and the partial results are merged; a prompt portion's
+    waves take their keys in ``n_splits`` parts where few waves stand behind long contexts."""
+    _masked_attention_checks("masked_attention_mfma", q, gate, gate_mode, k_pool, v_pool, sink,
+                             block_table, q_start, ctx_len, None, out, n_heads, n_kv_heads,
+                             key_width, value_width, page_size, max_ctx_len)
+    T = q.shape[0]
+    qs = _columns(q, "masked_attention_mfma: q")
+    gs = _columns(gate, "masked_attention_mfma: gate") if gate is not None else 0
+    if not masked_attention_mfma_covers(q.dtype, n_heads, n_kv_heads, key_width, value_width,
+                                        v_pool is None) or qs % 8 != 0 or q.data_ptr() % 16 != 0:
+        raise KernelUnavailable(f"masked_attention_mfma: bfloat16, (key, value) widths of "
+                                f"{MASKED_MFMA_SHAPES}, at most 32 heads a kv head, query rows "
+                                "aligned to 16 bytes")
+    n_seqs = ctx_len.shape[0]
+    max_pages = block_table.shape[1]
+    keys = max_pages * page_size
+    for bound in (window, chunk):
+        if bound > 0:
+            keys = min(keys, bound)
+    G = n_heads // n_kv_heads
+    lib = build.load("masked_attention")
+    decode = max_q_len == 1 and T == n_seqs
+    if decode:
+        span = keys + 31                      # the first chunk starts at a multiple of 32
+        blocks = n_splits if n_splits is not None else \
+            max(1, min(MASKED_DECODE_WORKGROUPS // max(1, n_seqs * n_kv_heads),
+                       (span + 255) // 256, 16))
+        if not 1 <= blocks <= 16:
+            raise KernelUnavailable("masked_attention_mfma: 1 to 16 workgroups a context")
+        wave_keys = ((span + 4 * blocks - 1) // (4 * blocks) + 31) // 32 * 32
+        parts, splits, n_tiles = blocks, 4 * blocks, n_seqs
+    else:
+        QT = max(1, MASKED_MFMA_ROWS // G)
+        n_tiles = (T + QT - 1) // QT + n_seqs
+        parts = n_splits
+        if parts is None:
+            waves = (T * n_heads + 31) // 32
+            parts = 1
+            while parts < MASKED_ROWS_MAX_PARTS and waves * parts < MASKED_ROWS_WAVES \
+                    and min(keys, max_ctx_len) >= 256 * parts:
+                parts *= 2
+        wave_keys, splits = 0, parts
+    ws_o = ws_ml = None
+    if decode or parts > 1:
+        ws_o = _workspace("masked_o", T * n_heads * splits * value_width, torch.float32, q.device)
+        ws_ml = _workspace("masked_ml", T * n_heads * splits * 2, torch.float32, q.device)
+    code = lib.zf_masked_attention_mfma(
+        _ptr(q), ctypes.c_longlong(qs), _ptr(gate), ctypes.c_longlong(gs), GATE_MODES[gate_mode],
+        _ptr(k_pool), _ptr(v_pool), _ptr(sink), _ptr(block_table), _ptr(q_start), _ptr(ctx_len),
+        _ptr(out), _ptr(ws_o), _ptr(ws_ml), ctypes.c_float(scale), ctypes.c_float(cap),
+        int(window), int(chunk), T, n_seqs, n_tiles, n_heads, n_kv_heads, key_width, value_width,
+        page_size, max_pages, 1 if decode else 0, parts, wave_keys, _stream())
+    _check(code, "masked_attention_mfma")

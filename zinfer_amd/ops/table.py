@@ -10,7 +10,8 @@ from dataclasses import dataclass
 from typing import Callable, Dict
 
 from . import (gated_act, moe_grouped, norm_add_norm, tied_attention_mfma)
-from . import (activation, head_products, masked_attention, norm_add_store, project_rows)
+from . import (activation, head_products, masked_attention, masked_attention_mfma,
+               norm_add_store, project_rows)
 from . import (embed_position, kv_rows_write, moe_down, moe_gate_up, moe_route, norm_rows,
                shared_kv_attention)
 from . import (advance_decode, apply_penalties, argmax, argmax_no_alloc, cast, check_tables,
@@ -94,6 +95,8 @@ KERNELS: Dict[str, KernelEntry] = {
     "masked_attention": KernelEntry(masked_attention, "masked_attention", "own: attention with a "
                                     "score cap, a learned sink, chunks or a window, a gate; the "
                                     "values a pool or the keys' leading columns"),
+    "masked_attention_mfma": KernelEntry(masked_attention_mfma, "masked_attention",
+                                         "own: the same attention in MFMA tiles (bfloat16)"),
     "head_products": KernelEntry(head_products, "masked_attention", "own: a matrix a head"),
     "mfma_loop": KernelEntry(mfma_loop, "gemm",
                              "own: MFMAs alone, the rate the tiled products are measured against"),

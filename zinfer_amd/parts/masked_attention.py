@@ -123,11 +123,11 @@ class MaskedGqaAttention(Mixer):
                          cache.page_size, segments)
         gate = proj[:, self.q_width + self.k_width + self.v_width:] if s.head_gate else None
         attn = step.scratch("attn", (T, s.n_heads * s.value_dim), act)
-        ops.masked_attention(q, gate, "head" if s.head_gate else None, cache.k_pool, cache.v_pool,
-                             self.sink, kv.block_table, step.q_start, step.ctx_len,
-                             step.seq_index, attn, float(s.scale), float(s.softcap or 0.0),
-                             int(s.window or 0), int(s.chunk or 0), s.n_heads, s.n_kv_heads,
-                             s.head_dim, s.value_dim, cache.page_size, step.max_ctx_len)
+        ops.attend_masked(q, gate, "head" if s.head_gate else None, cache.k_pool, cache.v_pool,
+                          self.sink, kv.block_table, step.q_start, step.ctx_len, step.seq_index,
+                          attn, float(s.scale), float(s.softcap or 0.0), int(s.window or 0),
+                          int(s.chunk or 0), s.n_heads, s.n_kv_heads, s.head_dim, s.value_dim,
+                          cache.page_size, step.max_q_len, step.max_ctx_len)
         self.o.forward(attn, residual, accumulate=accumulate, step=step if accumulate else None)
 
 
@@ -235,10 +235,10 @@ class LatentAttention(Mixer):
                                          rot_off=s.head_dim, skip=s.head_dim, dst_off=s.kv_rank,
                                          dst_hd=KW, **rot)])
         mixed = step.scratch("latent_mixed", (T, H * s.kv_rank), act)
-        ops.masked_attention(qa, None, None, cache.k_pool, None, None, kv.block_table,
-                             step.q_start, step.ctx_len, step.seq_index, mixed, float(s.scale),
-                             0.0, int(s.window or 0), int(s.chunk or 0), H, 1, KW, s.kv_rank,
-                             cache.page_size, step.max_ctx_len)
+        ops.attend_masked(qa, None, None, cache.k_pool, None, None, kv.block_table,
+                          step.q_start, step.ctx_len, step.seq_index, mixed, float(s.scale), 0.0,
+                          int(s.window or 0), int(s.chunk or 0), H, 1, KW, s.kv_rank,
+                          cache.page_size, step.max_q_len, step.max_ctx_len)
         gate = down[:, s.q_rank + KW:] if s.element_gate else None
         attn = step.scratch("attn", (T, H * s.value_dim), act)
         ops.head_products(mixed, 0, s.kv_rank, self.uv, gate, attn, 0, s.value_dim)
