@@ -748,10 +748,263 @@ def main_fezupel(args) -> int:
 
 
 
+# --------------------------------------------------------------------------- Lodenex beside Qwen3
+# Layer sizes that resemble served models; every shape is run beside the dense Qwen3 decoder of
+# the same width, heads, head size, depth and vocabulary whose gated feed-forward does the same
+# matrix work a token as the ungated one (three matrices of 2/3 the width instead of two).
+LODENEX_SHAPES = {
+    # grouped-query attention in chunks, values of their own
+    "gqa": dict(width=4096, heads=32, kv_heads=8, dim=128, ff=16384, layers=4, vocab=32768,
+                mixers=("attention",) * 4, chunk=8192),
+    # attention over a latent row of 128 + 64 numbers a token
+    "latent": dict(width=4096, heads=32, kv_heads=8, dim=128, ff=16384, layers=4, vocab=32768,
+                   mixers=("latent_attention",) * 4, window=4096, q_rank=1536, kv_rank=128,
+                   rot_dim=64),
+    # three chunked layers to one latent layer
+    "mixed": dict(width=4096, heads=32, kv_heads=8, dim=128, ff=16384, layers=4, vocab=32768,
+                  mixers=("attention", "attention", "latent_attention", "attention"), chunk=8192,
+                  window=4096, q_rank=1536, kv_rank=128, rot_dim=64),
+    # a latent of 512 + 64: wider than the MFMA attention kernels take (the 32-bit kernel runs)
+    "latent-512": dict(width=4096, heads=32, kv_heads=8, dim=128, ff=16384, layers=2, vocab=32768,
+                       mixers=("latent_attention",) * 2, window=4096, q_rank=1536, kv_rank=512,
+                       rot_dim=64),
+}
+
+
+def lodenex_config(sh: dict) -> dict:
+    def layer(kind):
+        if kind == "attention":
+            mixer = {"heads": sh["heads"], "kv_heads": sh["kv_heads"], "dim": sh["dim"],
+                     "vdim": sh["dim"], "scale": sh["dim"] ** -0.5, "softcap": 30.0,
+                     "mask": {"size": sh["chunk"]},
+                     "rot": {"base": 500000.0, "dims": sh["dim"] // 2,
+                             "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+        else:
+            mixer = {"heads": sh["heads"], "dim": sh["dim"], "rot_dim": sh["rot_dim"],
+                     "vdim": sh["dim"], "q_rank": sh["q_rank"], "kv_rank": sh["kv_rank"],
+                     "scale": (sh["dim"] + sh["rot_dim"]) ** -0.5, "mask": {"size": sh["window"]},
+                     "rot": {"base": 1000000.0, "dims": sh["rot_dim"],
+                             "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+        return {"type": kind, "mixer": mixer, "mlp": {"kind": "dense", "ff": sh["ff"]}}
+    return {"architecture": "Lodenex", "vocab": sh["vocab"], "width": sh["width"],
+            "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0}, "logit_softcap": 30.0,
+            "layers": [layer(k) for k in sh["mixers"]]}
+
+
+def lodenex_twin(sh: dict, max_positions: int) -> dict:
+    return dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3",
+                num_hidden_layers=sh["layers"], hidden_size=sh["width"],
+                num_attention_heads=sh["heads"], num_key_value_heads=sh["kv_heads"],
+                head_dim=sh["dim"], intermediate_size=sh["ff"] * 2 // 3 // 64 * 64,
+                vocab_size=sh["vocab"], rope_theta=1000000.0, rms_norm_eps=1e-6,
+                tie_word_embeddings=False, max_position_embeddings=max_positions,
+                torch_dtype="bfloat16")
+
+
+def _timed_graph(fn, inner: int = 10, repeats: int = 10) -> float:
+    """Seconds of one call of ``fn`` on the device: ``inner`` calls are recorded into one graph
+    (after two eager calls that settle work buffers) and the graph is replayed ``repeats`` times
+    between two events, so that what the host spends on a launch does not count: a decode step's
+    kernels run that way in the engine."""
+    import torch
+    fn()
+    fn()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(inner):
+            fn()
+    graph.replay()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(repeats):
+        graph.replay()
+    b.record()
+    b.synchronize()
+    return a.elapsed_time(b) * 1e-3 / (repeats * inner)
+
+
+def lodenex_kernels(sh: dict, T: int, ctx: int, mfma_rate: float, read_bw: float) -> dict:
+    """The new design's kernels alone beside the like kernels of the dense decoder, at ``T``
+    tokens of one sequence that holds ``ctx`` tokens (T = ctx: a prompt; T = 1 x 8 sequences: a
+    decode step), each with the fraction of its bound it reaches: matrix work against the MFMA
+    loop's rate (prompt) or bytes that must be read against the measured read stream (decode)."""
+    import torch
+    import zinfer_amd.ops as ops
+    dev = "cuda:0"
+    W, nH, nKV, hd, ff = sh["width"], sh["heads"], sh["kv_heads"], sh["dim"], sh["ff"]
+    bf = torch.bfloat16
+    decode = T == 1
+    n_seqs = 8 if decode else 1
+    rows = n_seqs * T
+    g = torch.Generator(device=dev).manual_seed(1)
+    rnd = lambda *shape: (torch.randn(shape, generator=g, device=dev) * 0.05).to(bf)
+    i32 = lambda a: torch.tensor(a, dtype=torch.int32, device=dev)
+    pages = (ctx + PAGE - 1) // PAGE
+    table = torch.arange(n_seqs * pages, dtype=torch.int32, device=dev).view(n_seqs, pages)
+    q_start = i32([i * T for i in range(n_seqs + 1)])
+    ctx_len = i32([ctx] * n_seqs)
+    seq_index = i32([i for i in range(n_seqs) for _ in range(T)])
+    positions = i32([ctx - T + t for _ in range(n_seqs) for t in range(T)])
+    slots = i32([(s * pages) * PAGE + ctx - T + t for s in range(n_seqs) for t in range(T)])
+    bound = "frac_of_read" if decode else "frac_of_mfma"
+    out = {}
+
+    def row(name, t_new, t_old, work_new, work_old):
+        rate = read_bw if decode else mfma_rate
+        r = {"lodenex_us": round(t_new * 1e6, 1), "lodenex_" + bound: round(work_new / t_new / rate, 4)}
+        if t_old is not None:
+            r.update({"qwen3_us": round(t_old * 1e6, 1),
+                      "qwen3_" + bound: round(work_old / t_old / rate, 4)})
+        out[name] = r
+
+    # ---- the dense decoder's attention at these heads
+    q = rnd(rows, nH * hd)
+    k_pool = rnd(n_seqs * pages, nKV * PAGE * hd)
+    v_pool = rnd(n_seqs * pages, nKV * PAGE * hd)
+    o = torch.empty((rows, nH * hd), dtype=bf, device=dev)
+    t_old = _timed_graph(lambda: ops.paged_attention(q, k_pool, v_pool, table, q_start, ctx_len,
+                                               seq_index, o, hd ** -0.5, 0, nH, nKV, hd, PAGE, T, ctx))
+    pairs = n_seqs * (ctx if decode else T * (T + 1) // 2)
+    old_work = n_seqs * ctx * nKV * 2 * hd * 2 if decode else 4.0 * pairs * hd * nH
+    if "attention" in sh["mixers"]:
+        gate = rnd(rows, nH)
+        sink = torch.zeros((nH,), device=dev)
+        t_new = _timed_graph(lambda: ops.attend_masked(q, gate, "head", k_pool, v_pool, sink, table, q_start,
+                                                 ctx_len, seq_index, o, hd ** -0.5, 30.0, 0, sh["chunk"],
+                                                 nH, nKV, hd, hd, PAGE, T, ctx))
+        row("attention", t_new, t_old, old_work, old_work)
+        # the projection's rows normed, rotated and stored, beside the dense decoder's kernel
+        width = (nH + 2 * nKV) * hd
+        proj = rnd(rows, width + nH)
+        gq, gk = torch.ones((nH * hd,), device=dev), torch.ones((nKV * hd,), device=dev)
+        freq = torch.rand((hd // 4,), generator=g, device=dev)
+        segs = [ops.RowSegment(0, nH * hd, q, gain=gq, eps=1e-6, hd=hd, rot_dims=hd // 2, freq=freq),
+                ops.RowSegment(nH * hd, nKV * hd, k_pool, gain=gk, eps=1e-6, hd=hd, rot_dims=hd // 2,
+                               freq=freq, pool_heads=nKV),
+                ops.RowSegment((nH + nKV) * hd, nKV * hd, v_pool, hd=hd, pool_heads=nKV)]
+        t_new = _timed_graph(lambda: ops.project_rows(proj, positions, slots, PAGE, segs))
+        qkv = rnd(rows, width)
+        cos = torch.rand((ctx + 1, hd // 2), generator=g, device=dev)
+        gh = torch.ones((hd,), device=dev)
+        t_qk = _timed_graph(lambda: ops.qk_norm_rope_kv_write(qkv, gh, gh, 1e-6, cos, cos, positions, slots,
+                                                        k_pool, v_pool, q, nH, nKV, hd, PAGE))
+        out["norm_rotate_store"] = {"lodenex_us": round(t_new * 1e6, 1), "qwen3_us": round(t_qk * 1e6, 1)}
+    if "latent_attention" in sh["mixers"]:
+        rank, dr = sh["kv_rank"], sh["rot_dim"]
+        KW = rank + dr
+        qa = rnd(rows, nH * KW)
+        lat_pool = rnd(n_seqs * pages, PAGE * KW)
+        mixed = torch.empty((rows, nH * rank), dtype=bf, device=dev)
+        seen = min(ctx, sh["window"])
+        t_new = _timed_graph(lambda: ops.attend_masked(qa, None, None, lat_pool, None, None, table, q_start,
+                                                 ctx_len, seq_index, mixed, KW ** -0.5, 0.0,
+                                                 sh["window"], 0, nH, 1, KW, rank, PAGE, T, ctx))
+        new_work = n_seqs * seen * KW * 2 if decode else 2.0 * pairs * (KW + rank) * nH
+        row("latent_attention", t_new, t_old, new_work, old_work)
+        # the two products a head around it
+        qfull = rnd(rows, nH * (hd + dr))
+        uk_t, uv = rnd(nH, rank, hd), rnd(nH, hd, rank)
+        attn = torch.empty((rows, nH * hd), dtype=bf, device=dev)
+        gate_e = rnd(rows, nH * hd)
+
+        def around():
+            ops.head_products(qfull, 0, hd + dr, uk_t, None, qa, 0, KW)
+            ops.head_products(mixed, 0, rank, uv, gate_e, attn, 0, hd)
+        t_hp = _timed_graph(around)
+        work = 2 * nH * rank * hd * 2 if decode else 2.0 * rows * 2 * nH * rank * hd
+        row("head_products", t_hp, None, work, None)
+    # ---- feed-forward: two matrices and an activation beside three of 2/3 the width
+    h = rnd(rows, W)
+    w_up, w_down = ops.pretile_weight(rnd(ff, W)), ops.pretile_weight(rnd(W, ff))
+    act = torch.empty((rows, ff), dtype=bf, device=dev)
+    branch = torch.zeros((rows, W), dtype=torch.float32, device=dev)
+
+    def plain_ff():
+        ops.gemm(h, w_up, act, w_tiled=True)
+        ops.activation(act, act, "gelu")
+        ops.gemm(act, w_down, branch, w_tiled=True)
+    t_new = _timed_graph(plain_ff)
+    inter = ff * 2 // 3 // 64 * 64
+    wgu = ops.pretile_weight(ops.interleave_gate_up(rnd(inter, W), rnd(inter, W)))
+    wd = ops.pretile_weight(rnd(W, inter))
+    act2 = torch.empty((rows, inter), dtype=bf, device=dev)
+
+    def gated_ff():
+        ops.gemm_swiglu(h, wgu, act2, w_tiled=True)
+        ops.gemm(act2, wd, branch, accumulate=True, w_tiled=True)
+    t_old = _timed_graph(gated_ff)
+    if decode:
+        row("feed_forward", t_new, t_old, 2 * ff * W * 2, 3 * inter * W * 2)
+    else:
+        row("feed_forward", t_new, t_old, 2.0 * rows * 2 * ff * W, 2.0 * rows * 3 * inter * W)
+    # ---- the norm behind a sublayer (adds, leaves the sum for the next product) beside an RMS
+    # norm that stores
+    x = torch.randn((rows, W), generator=g, device=dev)
+    gain = torch.ones((W,), device=dev)
+    normed = torch.empty((rows, W), dtype=bf, device=dev)
+    t_ln = _timed_graph(lambda: ops.norm_add_store(branch, gain, None, 1e-6, False, x, normed))
+    t_rms = _timed_graph(lambda: ops.rmsnorm(x, gain, 1e-6, normed))
+    out["norm"] = {"lodenex_us": round(t_ln * 1e6, 1), "qwen3_us": round(t_rms * 1e6, 1)}
+    return out
+
+
+def main_lodenex(args) -> int:
+    """Prefill and decode throughput of Lodenex shapes beside the dense Qwen3 decoder of equal
+    size, and the new kernels alone beside the like kernels of that decoder."""
+    import torch
+    import zinfer_amd.ops as ops
+    from zinfer_amd.config import entry_for
+    T, batch, prompt = args.prefill_tokens, args.batch, args.prompt_len
+    max_positions = max(T, prompt + args.steps + args.warmup + 64) + 64
+    read_bw = ops.measure_read_bandwidth("cuda:0")
+    mfma_rate = ops.measure_mfma_rate("cuda:0")
+    names = [args.lodenex_shape] if args.lodenex_shape else ["gqa", "latent", "mixed"]
+    shapes = {}
+    for name in names:
+        sh = LODENEX_SHAPES[name]
+        row = {"sizes": {k: (list(v) if isinstance(v, tuple) else v) for k, v in sh.items()}}
+        for label, raw in (("lodenex", lodenex_config(sh)), ("qwen3", lodenex_twin(sh, max_positions))):
+            cfg = entry_for(raw).config_type.from_dict(raw)
+            pool = batch * (prompt + args.steps + args.warmup + 64) + T + 256
+            llm = build_llm(raw, args.dtype, args.seed, pool, max(batch, 8),
+                            max_step_tokens=max(T, 2048), multi_step=args.multi_step)
+            t_pre = run_prefill(llm, cfg, T, args.seed + 1)
+            dt, mean_ctx = run_decode(llm, cfg, batch, prompt, args.steps, args.warmup, args.seed + 2)
+            row[label] = {"prefill_tokens_per_s": round(T / t_pre, 1), "prefill_ms": round(t_pre * 1e3, 3),
+                          "decode_tokens_per_s": round(batch * args.steps / dt, 1),
+                          "decode_ms_per_step": round(dt / args.steps * 1e3, 4),
+                          "decode_mean_context": round(mean_ctx, 1)}
+            drop(llm)
+        row["prefill_vs_qwen3"] = round(row["lodenex"]["prefill_tokens_per_s"]
+                                        / row["qwen3"]["prefill_tokens_per_s"], 3)
+        row["decode_vs_qwen3"] = round(row["lodenex"]["decode_tokens_per_s"]
+                                       / row["qwen3"]["decode_tokens_per_s"], 3)
+        if args.dtype == "bfloat16":
+            row["kernels_prefill"] = lodenex_kernels(sh, T, T, mfma_rate, read_bw)
+            row["kernels_decode"] = lodenex_kernels(sh, 1, prompt, mfma_rate, read_bw)
+        ops._workspaces.clear()
+        torch.cuda.empty_cache()
+        shapes[name] = row
+    first = shapes[names[0]]
+    print(json.dumps({
+        "metric": "lodenex_decode_tokens_per_s", "value": first["lodenex"]["decode_tokens_per_s"],
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": first["lodenex"]["decode_ms_per_step"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic", "config": {"model": f"Lodenex {names[0]} shape beside the dense Qwen3 "
+                                                 "decoder of equal size, random weights",
+                                        "batch": batch, "prompt_len": prompt, "prefill_tokens": T,
+                                        "parallelism": "single GPU"},
+        "measured_read_gbs": round(read_bw / 1e9, 1), "mfma_loop_tflops": round(mfma_rate / 1e12, 1),
+        "shapes": shapes}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "long-context", "fezupel"])
+    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "long-context", "fezupel", "lodenex"])
     ap.add_argument("--shape", default=None, choices=sorted(SHAPES),
                     help="layer sizes (default: 8b for decode, 14b for continuous, 32b for "
                          "long-context)")
@@ -787,6 +1040,8 @@ def main() -> int:
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--fezupel-shape", default=None, choices=sorted(FEZUPEL_SHAPES),
                     help="fezupel: only this shape (default: all of them)")
+    ap.add_argument("--lodenex-shape", default=None, choices=sorted(LODENEX_SHAPES),
+                    help="lodenex: only this shape (default: gqa, latent and mixed)")
     ap.add_argument("--no-run-graphs", action="store_true",
                     help="decode steps in a row replay one graph per step instead of one for the run")
     args = ap.parse_args()
@@ -795,7 +1050,8 @@ def main() -> int:
               "multi-GPU path")
         return 2
     return {"decode": main_decode, "continuous": main_continuous,
-            "long-context": main_long_context, "fezupel": main_fezupel}[args.workload](args)
+            "long-context": main_long_context, "fezupel": main_fezupel,
+            "lodenex": main_lodenex}[args.workload](args)
 
 
 if __name__ == "__main__":

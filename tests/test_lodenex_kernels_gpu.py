@@ -90,13 +90,42 @@ def test_head_products(dt, T, H, N, K):
         assert torch.equal(one[0], out[T // 2])
 
 
+@pytest.mark.parametrize("T, H, N, K", [(1, 3, 24, 16), (8, 32, 128, 128), (77, 6, 100, 48),
+                                        (300, 2, 192, 160)])
+def test_head_products_in_mfma_tiles(T, H, N, K):
+    """bfloat16 with k a multiple of 16 and rows aligned to 16 bytes: the MFMA form; outputs
+    that are no multiple of 32, tokens that are no multiple of 32, a gate, a row alone."""
+    dt = torch.bfloat16
+    a_hd, out_hd, a_off, out_off = K + 8, N + 3, 8, 1
+    a = _rand((T, a_off + H * a_hd + 8), 1, 1.0, dt)
+    w = _rand((H, N, K), 2, 1.0 / math.sqrt(K), dt)
+    gate = _rand((T, H * N), 3, 1.5, dt)
+    a64 = torch.stack([a[:, a_off + h * a_hd: a_off + h * a_hd + K] for h in range(H)], 1).double()
+    ref = torch.einsum("thk,hnk->thn", a64, w.double())
+    for g in (None, gate):
+        out = torch.zeros((T, out_off + H * out_hd + 2), dtype=dt, device=DEV)
+        ops.head_products(a.to(DEV), a_off, a_hd, w.to(DEV), None if g is None else g.to(DEV),
+                          out, out_off, out_hd)
+        got = torch.stack([out[:, out_off + h * out_hd: out_off + h * out_hd + N]
+                           for h in range(H)], 1)
+        want = ref if g is None else ref * torch.sigmoid(g.double()).view(T, H, N)
+        assert rel_err(got, want) < tol(dt)
+        assert float(out[:, :out_off].abs().max()) == 0.0
+        assert float(out[:, out_off + H * out_hd:].abs().max()) == 0.0
+        one = torch.zeros((1, out.shape[1]), dtype=dt, device=DEV)
+        ops.head_products(a[T // 2: T // 2 + 1].to(DEV), a_off, a_hd, w.to(DEV),
+                          None if g is None else g[T // 2: T // 2 + 1].to(DEV), one, out_off, out_hd)
+        assert torch.equal(one[0], out[T // 2])
+
+
 # ------------------------------------------------------------------------------ rows of a projection
+@pytest.mark.parametrize("d, dv, dims", [(10, 7, 6), (16, 8, 8)])     # plain rows; groups of 8
 @pytest.mark.parametrize("dt", DTYPES)
-def test_project_rows_norms_rotates_and_stores(dt):
+def test_project_rows_norms_rotates_and_stores(dt, d, dv, dims):
     """Three segments of one product: queries (normed over all heads at once, the first 6 of
     10 elements of a head rotated) into rows, keys the same into pages, values as they are into
     pages of their own width; positions up to a few thousand."""
-    T, H, G, d, dv, dims, ps = 9, 3, 2, 10, 7, 6, 4
+    T, H, G, ps = 9, 3, 2, 4
     src = _rand((T, H * d + G * d + G * dv + 5), 1, 1.5, dt)
     gq, gk = 1 + _rand((H * d,), 2, 0.3), 1 + _rand((G * d,), 3, 0.3)
     freqs = P.wavelength_scaled_frequencies(50.0, dims, {"factor": 4.0, "low": 1.0, "high": 3.0,
@@ -119,9 +148,9 @@ def test_project_rows_norms_rotates_and_stores(dt):
     assert rel_err(q.view(T, H, d), want_q) < lim
     want_k = P.rotate_leading(P.rms_norm(src[:, H * d:H * d + G * d], gk, 1e-5).view(T, G, d),
                               pos, freqs, dims)
-    got_k = kp.view(n_pages, G, ps, d)[slots // ps, :, slots % ps]
+    got_k = ops.masked_pool_rows(kp, G, ps, d)[slots // ps, :, slots % ps]
     assert rel_err(got_k, want_k) < lim
-    got_v = vp.view(n_pages, G, ps, dv)[slots // ps, :, slots % ps]
+    got_v = ops.masked_pool_rows(vp, G, ps, dv)[slots // ps, :, slots % ps]
     assert torch.equal(got_v.cpu(), src[:, H * d + G * d:H * d + G * d + G * dv].view(T, G, dv))
     # the elements behind the rotated ones pass through the norm alone
     assert rel_err(q.view(T, H, d)[..., dims:], want_q[..., dims:]) < tol(dt)
@@ -132,12 +161,13 @@ def test_project_rows_norms_rotates_and_stores(dt):
             assert float(kp[p].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("rank", [11, 12])       # a pool row of 15: plain rows; of 16: groups of 8
 @pytest.mark.parametrize("dt", DTYPES)
-def test_project_rows_latent_layout(dt):
+def test_project_rows_latent_layout(dt, rank):
     """A latent mixer's segments: the normed query latent into rows; the normed key latent and
     behind it the rotated shared part into one pool row; and of a query's heads the rotated
     part alone (``skip``), times a magnitude, behind the columns another kernel fills."""
-    T, rank_q, rank, dr, ps, H, d = 6, 9, 11, 4, 4, 3, 5
+    T, rank_q, dr, ps, H, d = 6, 9, 4, 4, 3, 5
     src = _rand((T, rank_q + rank + dr + 3), 5, 1.2, dt)
     gq, gc = 1 + _rand((rank_q,), 6, 0.3), 1 + _rand((rank,), 7, 0.3)
     freqs, mag = P.yarn_frequencies(11.0, dr, {"factor": 2.0, "original": 8, "fast": 3.0, "slow": 0.5})
@@ -152,7 +182,7 @@ def test_project_rows_latent_layout(dt):
         ops.RowSegment(rank_q + rank, dr, pool, rot_dims=dr, freq=f32, mag=mag, dst_off=rank,
                        dst_hd=rank + dr, pool_heads=1)])
     assert rel_err(cq, P.rms_norm(src[:, :rank_q], gq, 1e-3)) < tol(dt)
-    rows = pool.view(3, ps, rank + dr)[slots // ps, slots % ps]
+    rows = ops.masked_pool_rows(pool, 1, ps, rank + dr)[slots // ps, 0, slots % ps]
     assert rel_err(rows[:, :rank], P.rms_norm(src[:, rank_q:rank_q + rank], gc, 1e-3)) < tol(dt)
     want_r = P.rotate_leading(src[:, rank_q + rank:rank_q + rank + dr].view(T, 1, dr), pos, freqs, dr, mag)
     assert rel_err(rows[:, rank:], want_r.view(T, dr)) < tol(dt)
@@ -191,8 +221,9 @@ class Paged:
                 kp[page, :, :m] = self.k[s][i * ps:i * ps + m].transpose(0, 1)
                 if VW:
                     vp[page, :, :m] = self.v[s][i * ps:i * ps + m].transpose(0, 1)
-        self.k_pool = kp.view(n_pages, -1).to(DEV)
-        self.v_pool = vp.view(n_pages, -1).to(DEV) if VW else None
+        # (the kernels' own layout inside a block)
+        self.k_pool = ops.masked_pool_from_rows(kp).to(DEV)
+        self.v_pool = ops.masked_pool_from_rows(vp).to(DEV) if VW else None
         self.table = table.to(DEV)
 
 

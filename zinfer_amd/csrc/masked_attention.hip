@@ -9,8 +9,9 @@
 //                                                        has no key and no value (null: none)
 //   o_i  = sum_j a_ij v_j;  then o_i * sigmoid(gate) with one gate an element or one a head
 //
-// Keys lie in a pool [page, kv head, row, KW]; values in a pool of their own [page, kv head,
-// row, VW], or (no value pool) they are the first VW columns of the key rows: that is what
+// Keys lie in a pool of blocks [page, kv head] of page_size rows of KW elements; values in a
+// pool of their own (rows of VW elements), or (no value pool) they are the first VW columns of
+// the key rows: that is what
 // attention over a shared latent row looks like once the per-head key and value matrices have
 // been moved to the query's and the output's side (one kv head, a key row = the latent and the
 // rotated part, the value = the latent).
@@ -26,6 +27,14 @@
 //    latent attention's per-head matrices out of the attention), 32-bit sums in ascending k,
 //    with an optional gate sigmoid(g) on the output.
 #include "zf_common.h"
+
+// Where element d of row r lies in a block of page_size rows of W elements.  When W is a
+// multiple of 8 the block is laid out [W / 8][page_size][8]: the 16 bytes that hold 8 elements
+// of a row lie beside the same 16 bytes of the next row, so the lanes of a wave that load 16
+// bytes of 16 rows each (an MFMA operand) read 256 consecutive bytes.  Else plain rows.
+__host__ __device__ __forceinline__ size_t pool_at(int r, int d, int page_size, int W) {
+  return (W & 7) == 0 ? ((size_t)(d >> 3) * page_size + r) * 8 + (d & 7) : (size_t)r * W + d;
+}
 
 #define PR_MAX_SEGMENTS 4
 
@@ -50,15 +59,20 @@ struct RowSegments {
   int n;
 };
 
+#define PR_MAX_PAIRS 256      // a rotation's cosines and sines are kept in LDS: rot_dims <= 512
+
 template <typename T>
 __global__ __launch_bounds__(256) void project_rows_kernel(
     const T* __restrict__ src, long long src_stride, const int* __restrict__ positions,
     const int* __restrict__ slot_mapping, int page_size, RowSegments segs) {
 #pragma clang fp contract(off)
   __shared__ float red[16];
+  __shared__ float cs_t[PR_MAX_PAIRS], sn_t[PR_MAX_PAIRS];
   const int t = blockIdx.x;
   const T* row = src + (size_t)t * src_stride;
   const float pos = (float)positions[t];
+  const float* have = nullptr;          // the frequencies the tables in LDS were made from
+  float have_mag = 0.f;
   for (int si = 0; si < segs.n; ++si) {
     const RowSegment& g = segs.s[si];
     const T* x = row + g.src_off;
@@ -81,6 +95,20 @@ __global__ __launch_bounds__(256) void project_rows_kernel(
       pool_row = slot % page_size;
     }
     const int half = g.rot_dims / 2;
+    // the token's cosine and sine a pair, once for all heads (and for the next segment, if it
+    // turns by the same frequencies)
+    if (half > 0 && (have != g.freq || have_mag != g.mag)) {
+      __syncthreads();
+      for (int j = threadIdx.x; j < half; j += blockDim.x) {
+        float sn, cs;
+        sincosf(pos * g.freq[j], &sn, &cs);
+        cs_t[j] = cs * g.mag;
+        sn_t[j] = sn * g.mag;
+      }
+      __syncthreads();
+      have = g.freq;
+      have_mag = g.mag;
+    }
     for (int i = threadIdx.x; i < g.width; i += blockDim.x) {
       const int head = i / g.hd, d = i % g.hd;
       if (d < g.skip) continue;
@@ -92,16 +120,13 @@ __global__ __launch_bounds__(256) void project_rows_kernel(
         const int pi = first ? i + half : i - half;
         float b = load_as_float<T>(x + pi);
         if (g.gain != nullptr) b = b * inv * g.gain[pi];
-        const float ang = pos * g.freq[first ? r : r - half];
-        float sn, cs;
-        sincosf(ang, &sn, &cs);
-        cs = cs * g.mag;
-        sn = sn * g.mag;
+        const int j = first ? r : r - half;
+        const float cs = cs_t[j], sn = sn_t[j];
         a = first ? a * cs - b * sn : a * cs + b * sn;
       }
       if (g.to_pool) {
-        T* o = (T*)g.dst + ((pool_base + head) * page_size + pool_row) * (size_t)g.dst_hd
-               + g.dst_off + (d - g.skip);
+        T* o = (T*)g.dst + (pool_base + head) * page_size * (size_t)g.dst_hd
+               + pool_at(pool_row, g.dst_off + (d - g.skip), page_size, g.dst_hd);
         store_from_float<T>(o, a);
       } else {
         T* o = (T*)g.dst + (size_t)t * g.dst_stride + g.dst_off + (size_t)head * g.dst_hd
@@ -134,7 +159,8 @@ extern "C" int zf_project_rows(const void* src, int dtype, long long src_stride,
     g.dst_stride = strides[i];
     if (g.width <= 0 || g.hd <= 0 || g.width % g.hd != 0 || g.rot_dims < 0 || g.rot_dims % 2 != 0
         || g.rot_off < 0 || g.rot_off + g.rot_dims > g.hd || g.skip < 0 || g.skip >= g.hd
-        || (g.rot_dims > 0 && g.freq == nullptr) || g.dst == nullptr
+        || (g.rot_dims > 0 && g.freq == nullptr) || g.rot_dims > 2 * PR_MAX_PAIRS
+        || g.dst == nullptr
         || (g.to_pool && (slot_mapping == nullptr || page_size <= 0 || g.pool_heads <= 0)))
       return -2;
   }
@@ -178,7 +204,7 @@ __global__ __launch_bounds__(MA_MAX_WAVES * ZF_WAVE) void masked_attention_kerne
   float* vs = ks + KC * ldk;                       // [KC][ldv] when the values have a pool
   float* qs = vs + (v_pool != nullptr ? KC * ldv : 0);   // [n_waves][KW]
   float* ps = qs + n_waves * KW;                   // [n_waves][ZF_WAVE]
-  int* rows = (int*)(ps + n_waves * ZF_WAVE);      // [KC]: row of each key in the pools
+  int* rows = (int*)(ps + n_waves * ZF_WAVE);      // [KC]: block of each key in the pools
 
   const int t = blockIdx.x, kvh = blockIdx.y;
   const int G = a.nH / a.nKV;
@@ -216,18 +242,19 @@ __global__ __launch_bounds__(MA_MAX_WAVES * ZF_WAVE) void masked_attention_kerne
     __syncthreads();                               // the tiles of the chunk before are done with
     if ((int)threadIdx.x < KC) {
       const int key = base + threadIdx.x;
-      rows[threadIdx.x] = key <= pos
-          ? (table[key / a.page_size] * a.nKV + kvh) * a.page_size + key % a.page_size : -1;
+      rows[threadIdx.x] = key <= pos ? table[key / a.page_size] * a.nKV + kvh : -1;
     }
     __syncthreads();
     for (int i = threadIdx.x; i < nk * KW; i += blockDim.x) {
       const int j = i / KW, d = i % KW;
-      ks[j * ldk + d] = load_as_float<T>(k_pool + (size_t)rows[j] * KW + d);
+      ks[j * ldk + d] = load_as_float<T>(k_pool + (size_t)rows[j] * a.page_size * KW
+                                         + pool_at((base + j) % a.page_size, d, a.page_size, KW));
     }
     if (v_pool != nullptr)
       for (int i = threadIdx.x; i < nk * VW; i += blockDim.x) {
         const int j = i / VW, d = i % VW;
-        vs[j * ldv + d] = load_as_float<T>(v_pool + (size_t)rows[j] * VW + d);
+        vs[j * ldv + d] = load_as_float<T>(v_pool + (size_t)rows[j] * a.page_size * VW
+                                           + pool_at((base + j) % a.page_size, d, a.page_size, VW));
       }
     __syncthreads();
     float sc = -INFINITY;
@@ -382,6 +409,76 @@ __global__ __launch_bounds__(256) void head_products_kernel(
   }
 }
 
+// The same in MFMA tiles for bfloat16 operands (K a multiple of 16, rows aligned to 16 bytes):
+// a wave takes 32 outputs x 32 tokens of one head, D = W_h tile (32 x K) times a^T (K x 32), both
+// operands straight from memory into v_mfma_f32_32x32x16_bf16, k upwards in one accumulator; a
+// lane ends with four runs of four consecutive outputs of one token.  The four waves of a
+// workgroup take four tiles of outputs.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 hp_bf16x8_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float hp_f32x16_t;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t hp_u32x4_t;
+
+__global__ __launch_bounds__(256) void head_products_mfma_kernel(
+    const bf16_t* __restrict__ a, long long a_stride, int a_off, int a_hd,
+    const bf16_t* __restrict__ w, const bf16_t* __restrict__ gate, long long gate_stride,
+    bf16_t* __restrict__ out, long long out_stride, int out_off, int out_hd, int n_tok, int N,
+    int K) {
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int c = lane % 32, hl = lane / 32;
+  const int t0 = blockIdx.x * 32, h = blockIdx.y, n0 = (blockIdx.z * 4 + wave) * 32;
+  if (n0 >= N) return;
+  const int t = t0 + c, n = n0 + c;
+  const bool t_ok = t < n_tok, n_ok = n < N;
+  const bf16_t* arow = a + (size_t)(t_ok ? t : 0) * a_stride + a_off + (size_t)h * a_hd;
+  const bf16_t* wrow = w + ((size_t)h * N + (n_ok ? n : 0)) * K;
+  hp_f32x16_t acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+  // four k-steps' operands are asked for before the first of their products
+  for (int k0 = 0; k0 < K; k0 += 64) {
+    hp_u32x4_t av[4], wv[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      av[u] = hp_u32x4_t{0u, 0u, 0u, 0u};
+      wv[u] = hp_u32x4_t{0u, 0u, 0u, 0u};
+      const int k = k0 + 16 * u + 8 * hl;
+      if (k < K) {
+        if (t_ok) av[u] = *(const hp_u32x4_t*)(arow + k);
+        if (n_ok) wv[u] = *(const hp_u32x4_t*)(wrow + k);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (k0 + 16 * u < K)
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const hp_bf16x8_t*)&wv[u],
+                                                      *(const hp_bf16x8_t*)&av[u], acc, 0, 0, 0);
+  }
+  if (!t_ok) return;
+  // acc[r] is output n0 + 8 (r / 4) + 4 hl + r % 4 of token t
+  bf16_t* orow = out + (size_t)t * out_stride + out_off + (size_t)h * out_hd;
+  const bf16_t* grow = gate != nullptr ? gate + (size_t)t * gate_stride + (size_t)h * N : nullptr;
+  // runs of four outputs as one 8-byte store where the rows allow it
+  const bool wide = (N & 3) == 0 && (((size_t)t * out_stride + out_off + (size_t)h * out_hd) & 3) == 0
+      && ((uintptr_t)out & 7) == 0;
+#pragma unroll
+  for (int r4 = 0; r4 < 4; ++r4) {
+    const int o = n0 + 8 * r4 + 4 * hl;
+    float v[4];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      v[x] = acc[4 * r4 + x];
+      if (grow != nullptr && o + x < N) v[x] *= 1.0f / (1.0f + expf(-bf16_to_float(grow[o + x])));
+    }
+    if (wide && o < N) {
+      *(uint2*)(orow + o) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+    } else {
+#pragma unroll
+      for (int x = 0; x < 4; ++x)
+        if (o + x < N) orow[o + x] = float_to_bf16(v[x]);
+    }
+  }
+}
+
 extern "C" int zf_head_products(const void* a, int dtype, long long a_stride, int a_off, int a_hd,
                                 const void* w, int w_dtype, const void* gate,
                                 long long gate_stride, void* out, long long out_stride,
@@ -389,6 +486,14 @@ extern "C" int zf_head_products(const void* a, int dtype, long long a_stride, in
                                 hipStream_t stream) {
   if (T <= 0) return 0;
   if (H <= 0 || N <= 0 || K <= 0 || a_hd < K || out_hd < N) return -2;
+  if (dtype == ZF_BF16 && w_dtype == ZF_BF16 && K % 16 == 0 && a_stride % 8 == 0 && a_off % 8 == 0
+      && a_hd % 8 == 0 && (uintptr_t)a % 16 == 0 && (uintptr_t)w % 16 == 0) {
+    dim3 mgrid((T + 31) / 32, H, (N + 127) / 128);
+    hipLaunchKernelGGL(head_products_mfma_kernel, mgrid, dim3(256), 0, stream, (const bf16_t*)a,
+                       a_stride, a_off, a_hd, (const bf16_t*)w, (const bf16_t*)gate, gate_stride,
+                       (bf16_t*)out, out_stride, out_off, out_hd, T, N, K);
+    ZF_CHECK_LAUNCH();
+  }
   dim3 grid((T + HP_TOK - 1) / HP_TOK, H, (N + HP_OUT - 1) / HP_OUT);
 #define HP_LAUNCH(TA, TWT)                                                                      \
   hipLaunchKernelGGL((head_products_kernel<TA, TWT>), grid, dim3(256), 0, stream, (const TA*)a, \
@@ -406,7 +511,8 @@ extern "C" int zf_head_products(const void* a, int dtype, long long a_stride, in
 //  bfloat16 MFMA kernels: waves on their own
 // =====================================================================================
 // The same attention in v_mfma_f32_32x32x16_bf16 tiles, for key rows of KD and value rows of VD
-// elements (KD a multiple of 16, VD of 32) and at most 32 query heads a kv head.  A wave takes
+// elements (KD a multiple of 16, VD of 32; the pools in the [W / 8][page_size][8] form of
+// pool_at) and at most 32 query heads a kv head.  A wave takes
 // 32 rows, (position, head of the group) pairs of one sequence, and walks the keys those rows
 // see in chunks of 32, on its own: no barrier between waves anywhere.  A lane loads, for its
 // key of the chunk, the 8 values that its operand of S^T = K Q^T needs straight from the pool
@@ -489,8 +595,10 @@ __global__ __launch_bounds__(256, 2) void masked_attention_wave_kernel(
   } else {
     split = blockIdx.z;
     n_splits = gridDim.z;
+    // the last tiles of a sequence walk the most keys: they are handed out first, so that the
+    // grid does not end on its longest workgroups
     s = 0;
-    int tile = blockIdx.x;
+    int tile = (int)gridDim.x - 1 - (int)blockIdx.x;
     for (; s < a.n_seqs; ++s) {
       const int n = (q_start[s + 1] - q_start[s] + a.QT - 1) / a.QT;
       if (tile < n) break;
@@ -558,20 +666,22 @@ __global__ __launch_bounds__(256, 2) void masked_attention_wave_kernel(
   // every i, of its value row the same
   mw_u32x4_t kf[KD / 16];
   mw_u32x4_t vf[TIED ? 1 : VD / 16];
+  // the block [page, kv head] of this lane's key, in rows: its row there is key % page_size
   auto row_of = [&](int base, bool& ok) {
     const int key = base + c;
     ok = key >= k_first && key < k_end;          // (pages before k_first may have gone back)
     size_t prow = 0;
-    if (ok) prow = ((size_t)table[key / page_size] * nKV + kvh) * page_size + key % page_size;
+    if (ok) prow = ((size_t)table[key / page_size] * nKV + kvh) * page_size;
     return prow;
   };
   auto fetch_k = [&](int base) {
     bool ok;
     const size_t prow = row_of(base, ok);
+    const int r = (base + c) % page_size;
 #pragma unroll
     for (int i = 0; i < KD / 16; ++i) {
       mw_u32x4_t v = {0u, 0u, 0u, 0u};
-      if (ok) v = *(const mw_u32x4_t*)(k_pool + prow * KD + 16 * i + 8 * hl);
+      if (ok) v = *(const mw_u32x4_t*)(k_pool + prow * KD + ((size_t)(2 * i + hl) * page_size + r) * 8);
       kf[i] = v;
     }
   };
@@ -579,10 +689,11 @@ __global__ __launch_bounds__(256, 2) void masked_attention_wave_kernel(
     if constexpr (!TIED) {
       bool ok;
       const size_t prow = row_of(base, ok);
+      const int r = (base + c) % page_size;
 #pragma unroll
       for (int i = 0; i < VD / 16; ++i) {
         mw_u32x4_t v = {0u, 0u, 0u, 0u};
-        if (ok) v = *(const mw_u32x4_t*)(v_pool + prow * VD + 16 * i + 8 * hl);
+        if (ok) v = *(const mw_u32x4_t*)(v_pool + prow * VD + ((size_t)(2 * i + hl) * page_size + r) * 8);
         vf[i] = v;
       }
     }

@@ -1932,8 +1932,8 @@ class RowSegment:
     angles position * ``freq`` [rot_dims / 2] (float32), cosine and sine times ``mag``; the
     elements of a head below ``skip`` are not written.  The rest goes to ``dst``: plain rows
     [T, ...] where head h starts at column dst_off + h * dst_hd (dst_hd None: hd - skip), or
-    (``pool_heads`` given) a pool [page, kv head, row, dst_hd] at the token's slot, from column
-    dst_off of the pool row on."""
+    (``pool_heads`` given) a pool of blocks [page, kv head] of rows of dst_hd elements (laid out as
+    ``masked_pool_from_rows`` says) at the token's slot, from column dst_off of the row on."""
 
     def __init__(self, src_off: int, width: int, dst: torch.Tensor, *, gain=None, eps: float = 0.0,
                  hd: Optional[int] = None, rot_off: int = 0, rot_dims: int = 0, freq=None,
@@ -2008,6 +2008,27 @@ def project_rows(src: torch.Tensor, positions: torch.Tensor, slot_mapping: Optio
         (ctypes.c_longlong * len(strides))(*strides), _stream()), "project_rows")
 
 
+def masked_pool_from_rows(rows: torch.Tensor) -> torch.Tensor:
+    """A pool [pages, heads * page_size * W] in the layout ``project_rows`` writes and the
+    ``masked_attention`` kernels read, from rows [pages, heads, page_size, W]: with W a multiple
+    of 8 a block [page, head] is laid out [W / 8][page_size][8] (the 16 bytes of 8 elements of
+    a row beside the same 16 bytes of the next row: what 16 lanes of a wave load for an MFMA
+    operand is 256 consecutive bytes), else in plain rows."""
+    P, H, ps, W = rows.shape
+    if W % 8 == 0:
+        rows = rows.view(P, H, ps, W // 8, 8).permute(0, 1, 3, 2, 4)
+    return rows.contiguous().view(P, H * ps * W)
+
+
+def masked_pool_rows(pool: torch.Tensor, n_heads: int, page_size: int, width: int) -> torch.Tensor:
+    """The rows [pages, heads, page_size, W] a pool of that layout holds (a copy)."""
+    P = pool.shape[0]
+    if width % 8 == 0:
+        return pool.view(P, n_heads, width // 8, page_size, 8).permute(0, 1, 3, 2, 4) \
+            .reshape(P, n_heads, page_size, width)
+    return pool.view(P, n_heads, page_size, width).clone()
+
+
 GATE_MODES = {None: 0, "element": 1, "head": 2}
 
 
@@ -2057,9 +2078,9 @@ def masked_attention(q: torch.Tensor, gate: Optional[torch.Tensor], gate_mode: O
                      out: torch.Tensor, scale: float, cap: float, window: int, chunk: int,
                      n_heads: int, n_kv_heads: int, key_width: int, value_width: int,
                      page_size: int, max_ctx_len: int) -> None:
-    """Causal grouped-query attention over paged pools: keys [page, kv head, row, key width],
-    values [page, kv head, row, value width], or with ``v_pool`` None the first ``value_width``
-    columns of the key rows.  Token t of sequence s = seq_index[t] has position p = ctx_len[s] -
+    """Causal grouped-query attention over paged pools of blocks [page, kv head] of rows (laid
+    out as ``masked_pool_from_rows`` says): keys of ``key_width``, values of ``value_width``
+    elements, or with ``v_pool`` None the first ``value_width`` columns of the key rows.  Token t of sequence s = seq_index[t] has position p = ctx_len[s] -
     q_len[s] + (t - q_start[s]) and reads the keys j <= p with p - j < window (window > 0) and
     floor(j / chunk) == floor(p / chunk) (chunk > 0).  Scores are scale * q . k, then with
     cap > 0 cap * tanh(score / cap).  ``sink`` [nH] float32: the soft-max's denominator holds
