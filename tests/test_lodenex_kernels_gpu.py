@@ -119,14 +119,15 @@ def test_head_products_in_mfma_tiles(T, H, N, K):
 
 
 # ------------------------------------------------------------------------------ rows of a projection
-@pytest.mark.parametrize("d, dv, dims", [(10, 7, 6), (16, 8, 8)])     # plain rows; groups of 8
+# plain rows; pools in groups of 8; everything in groups of 8 (the kernel that moves 16 bytes)
+@pytest.mark.parametrize("d, dv, dims", [(10, 7, 6), (16, 8, 8), (32, 16, 16)])
 @pytest.mark.parametrize("dt", DTYPES)
 def test_project_rows_norms_rotates_and_stores(dt, d, dv, dims):
     """Three segments of one product: queries (normed over all heads at once, the first 6 of
     10 elements of a head rotated) into rows, keys the same into pages, values as they are into
     pages of their own width; positions up to a few thousand."""
     T, H, G, ps = 9, 3, 2, 4
-    src = _rand((T, H * d + G * d + G * dv + 5), 1, 1.5, dt)
+    src = _rand((T, H * d + G * d + G * dv + (8 if d == 32 else 5)), 1, 1.5, dt)
     gq, gk = 1 + _rand((H * d,), 2, 0.3), 1 + _rand((G * d,), 3, 0.3)
     freqs = P.wavelength_scaled_frequencies(50.0, dims, {"factor": 4.0, "low": 1.0, "high": 3.0,
                                                         "original": 20})
@@ -161,14 +162,16 @@ def test_project_rows_norms_rotates_and_stores(dt, d, dv, dims):
             assert float(kp[p].abs().max()) == 0.0
 
 
-@pytest.mark.parametrize("rank", [11, 12])       # a pool row of 15: plain rows; of 16: groups of 8
+# a pool row of 15: plain rows; of 16: groups of 8; everything in groups of 8
+@pytest.mark.parametrize("rank_q, rank, dr, d, extra", [(9, 11, 4, 5, 3), (9, 12, 4, 5, 3),
+                                                        (16, 24, 16, 8, 8)])
 @pytest.mark.parametrize("dt", DTYPES)
-def test_project_rows_latent_layout(dt, rank):
+def test_project_rows_latent_layout(dt, rank_q, rank, dr, d, extra):
     """A latent mixer's segments: the normed query latent into rows; the normed key latent and
     behind it the rotated shared part into one pool row; and of a query's heads the rotated
     part alone (``skip``), times a magnitude, behind the columns another kernel fills."""
-    T, rank_q, dr, ps, H, d = 6, 9, 4, 4, 3, 5
-    src = _rand((T, rank_q + rank + dr + 3), 5, 1.2, dt)
+    T, ps, H = 6, 4, 3
+    src = _rand((T, rank_q + rank + dr + extra), 5, 1.2, dt)
     gq, gc = 1 + _rand((rank_q,), 6, 0.3), 1 + _rand((rank,), 7, 0.3)
     freqs, mag = P.yarn_frequencies(11.0, dr, {"factor": 2.0, "original": 8, "fast": 3.0, "slow": 0.5})
     f32 = freqs.to(torch.float32).to(DEV)

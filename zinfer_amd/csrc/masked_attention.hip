@@ -137,6 +137,112 @@ __global__ __launch_bounds__(256) void project_rows_kernel(
   }
 }
 
+// The same for bfloat16 rows whose segments are made of whole groups of 8 elements (head
+// sizes, rotated ranges and their halves, offsets and strides all multiples of 8): a thread
+// takes 8 consecutive elements, 16 bytes in and 16 bytes out (a pool's 8 elements of a row are
+// consecutive).  The same arithmetic as the kernel above (the norm's partial sums are added in
+// another order).
+__device__ __forceinline__ void pr_unpack8(const uint4& v, float (&f)[8]) {
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f[2 * i] = __uint_as_float(w[i] << 16);
+    f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
+
+__global__ __launch_bounds__(256) void project_rows_vec8_kernel(
+    const bf16_t* __restrict__ src, long long src_stride, const int* __restrict__ positions,
+    const int* __restrict__ slot_mapping, int page_size, RowSegments segs) {
+#pragma clang fp contract(off)
+  __shared__ float red[16];
+  __shared__ float cs_t[PR_MAX_PAIRS], sn_t[PR_MAX_PAIRS];
+  const int t = blockIdx.x;
+  const bf16_t* row = src + (size_t)t * src_stride;
+  const float pos = (float)positions[t];
+  const float* have = nullptr;
+  float have_mag = 0.f;
+  for (int si = 0; si < segs.n; ++si) {
+    const RowSegment& g = segs.s[si];
+    const bf16_t* x = row + g.src_off;
+    const int n8 = g.width / 8;
+    float inv = 1.f;
+    if (g.gain != nullptr) {
+      float ss = 0.f;
+      for (int c = threadIdx.x; c < n8; c += blockDim.x) {
+        float f[8];
+        pr_unpack8(*(const uint4*)(x + 8 * c), f);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss += f[e] * f[e];
+      }
+      ss = block_sum(ss, red);
+      inv = 1.0f / sqrtf(ss / (float)g.width + g.eps);
+    }
+    size_t pool_base = 0;
+    int pool_row = 0;
+    if (g.to_pool) {
+      const int slot = slot_mapping[t];
+      if (slot < 0) continue;
+      pool_base = (size_t)(slot / page_size) * g.pool_heads;
+      pool_row = slot % page_size;
+    }
+    const int half = g.rot_dims / 2;
+    if (half > 0 && (have != g.freq || have_mag != g.mag)) {
+      __syncthreads();
+      for (int j = threadIdx.x; j < half; j += blockDim.x) {
+        float sn, cs;
+        sincosf(pos * g.freq[j], &sn, &cs);
+        cs_t[j] = cs * g.mag;
+        sn_t[j] = sn * g.mag;
+      }
+      __syncthreads();
+      have = g.freq;
+      have_mag = g.mag;
+    }
+    for (int c = threadIdx.x; c < n8; c += blockDim.x) {
+      const int i = 8 * c;
+      const int head = i / g.hd, d = i % g.hd;
+      if (d < g.skip) continue;
+      float a[8];
+      pr_unpack8(*(const uint4*)(x + i), a);
+      if (g.gain != nullptr) {
+        const float4 g0 = *(const float4*)(g.gain + i), g1 = *(const float4*)(g.gain + i + 4);
+        const float gg[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) a[e] = a[e] * inv * gg[e];
+      }
+      const int r = d - g.rot_off;
+      if (r >= 0 && r < g.rot_dims) {
+        const bool first = r < half;
+        const int pi = first ? i + half : i - half;
+        float b[8];
+        pr_unpack8(*(const uint4*)(x + pi), b);
+        if (g.gain != nullptr) {
+          const float4 g0 = *(const float4*)(g.gain + pi), g1 = *(const float4*)(g.gain + pi + 4);
+          const float gg[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+#pragma unroll
+          for (int e = 0; e < 8; ++e) b[e] = b[e] * inv * gg[e];
+        }
+        const int j = first ? r : r - half;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float cs = cs_t[j + e], sn = sn_t[j + e];
+          a[e] = first ? a[e] * cs - b[e] * sn : a[e] * cs + b[e] * sn;
+        }
+      }
+      bf16_t* o;
+      if (g.to_pool)
+        o = (bf16_t*)g.dst + (pool_base + head) * page_size * (size_t)g.dst_hd
+            + pool_at(pool_row, g.dst_off + (d - g.skip), page_size, g.dst_hd);
+      else
+        o = (bf16_t*)g.dst + (size_t)t * g.dst_stride + g.dst_off + (size_t)head * g.dst_hd
+            + (d - g.skip);
+      *(uint4*)o = make_uint4(pack_bf16x2(a[0], a[1]), pack_bf16x2(a[2], a[3]),
+                              pack_bf16x2(a[4], a[5]), pack_bf16x2(a[6], a[7]));
+    }
+  }
+}
+
 // ints: 11 a segment (src_off, width, hd, rot_off, rot_dims, skip, to_pool, dst_off, dst_hd,
 // pool_heads, 0); floats: 2 a segment (eps, mag); ptrs: 3 a segment (gain, freq, dst);
 // strides: 1 a segment
@@ -163,6 +269,18 @@ extern "C" int zf_project_rows(const void* src, int dtype, long long src_stride,
         || g.dst == nullptr
         || (g.to_pool && (slot_mapping == nullptr || page_size <= 0 || g.pool_heads <= 0)))
       return -2;
+  }
+  bool vec8 = dtype == ZF_BF16 && src_stride % 8 == 0 && (uintptr_t)src % 16 == 0;
+  for (int i = 0; i < n_segs && vec8; ++i) {
+    const RowSegment& g = segs.s[i];
+    vec8 = g.src_off % 8 == 0 && g.hd % 8 == 0 && g.rot_off % 8 == 0 && g.rot_dims % 16 == 0
+        && g.skip % 8 == 0 && g.dst_off % 8 == 0 && g.dst_hd % 8 == 0 && (uintptr_t)g.dst % 16 == 0
+        && (g.to_pool || g.dst_stride % 8 == 0) && (g.gain == nullptr || (uintptr_t)g.gain % 16 == 0);
+  }
+  if (vec8) {
+    hipLaunchKernelGGL(project_rows_vec8_kernel, dim3(T), dim3(256), 0, stream,
+                       (const bf16_t*)src, src_stride, positions, slot_mapping, page_size, segs);
+    ZF_CHECK_LAUNCH();
   }
   if (dtype == ZF_F32)
     hipLaunchKernelGGL(project_rows_kernel<float>, dim3(T), dim3(256), 0, stream,

@@ -2209,7 +2209,7 @@ def masked_attention_mfma(q, gate, gate_mode, k_pool, v_pool, sink, block_table,
         span = keys + 31                      # the first chunk starts at a multiple of 32
         blocks = n_splits if n_splits is not None else \
             max(1, min(MASKED_DECODE_WORKGROUPS // max(1, n_seqs * n_kv_heads),
-                       (span + 255) // 256, 16))
+                       (span + 383) // 384, 16))
         if not 1 <= blocks <= 16:
             raise KernelUnavailable("masked_attention_mfma: 1 to 16 workgroups a context")
         wave_keys = ((span + 4 * blocks - 1) // (4 * blocks) + 31) // 32 * 32
