@@ -308,7 +308,8 @@ def test_attention_against_plain(dt, case):
 
 @pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("H, KW, VW, ps, n, window", [(3, 28, 24, 4, 50, 5), (7, 13, 11, 16, 40, 1),
-                                                       (4, 160, 128, 16, 90, 40), (2, 96, 48, 8, 300, 0)])
+                                                       (4, 160, 128, 16, 90, 40), (2, 96, 48, 8, 300, 0),
+                                                       (32, 576, 512, 16, 70, 0), (20, 1200, 8, 16, 40, 7)])
 def test_values_that_are_the_keys_leading_columns(dt, H, KW, VW, ps, n, window):
     """No value pool: one kv head whose value is the first VW columns of its key row."""
     pg = Paged([n, 7], 1, KW, 0, ps, dt, 9)

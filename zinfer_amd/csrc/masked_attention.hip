@@ -327,7 +327,7 @@ __global__ __launch_bounds__(MA_MAX_WAVES * ZF_WAVE) void masked_attention_kerne
   const int t = blockIdx.x, kvh = blockIdx.y;
   const int G = a.nH / a.nKV;
   const int wave = threadIdx.x / ZF_WAVE, lane = threadIdx.x % ZF_WAVE;
-  const int g = blockIdx.z * MA_MAX_WAVES + wave;  // this wave's head within the group
+  const int g = blockIdx.z * n_waves + wave;       // this wave's head within the group
   const bool live = g < G;
   const int h = kvh * G + (live ? g : 0);
   const int s = seq_index[t];
@@ -421,11 +421,11 @@ __global__ __launch_bounds__(MA_MAX_WAVES * ZF_WAVE) void masked_attention_kerne
   }
 }
 
-// floats a key of a chunk takes in LDS, and the chunk that fits 40 KB beside the queries
+// floats a key of a chunk takes in LDS, and the chunk that fits 60 KB beside the queries
 static int ma_chunk_keys(int KW, int VW, bool v_pool, int n_waves) {
   const long per_key = (KW + 1) + (v_pool ? VW + 1 : 0) + 1;
   const long fixed = (long)n_waves * (KW + ZF_WAVE);
-  long kc = (40 * 1024 / 4 - fixed) / per_key;
+  long kc = (60 * 1024 / 4 - fixed) / per_key;
   if (kc > ZF_WAVE) kc = ZF_WAVE;
   return (int)kc;
 }
@@ -444,14 +444,16 @@ extern "C" int zf_masked_attention(const void* q, long long q_stride, const void
       || gate_mode < 0 || gate_mode > 2 || window < 0 || chunk < 0 || cap < 0.f)
     return -2;
   const int G = nH / nKV;
-  const int n_waves = G < MA_MAX_WAVES ? G : MA_MAX_WAVES;
+  // a wave a head, up to 16; fewer where wide rows would leave no room for a chunk of keys
+  int n_waves = G < MA_MAX_WAVES ? G : MA_MAX_WAVES;
+  while (n_waves > 1 && ma_chunk_keys(KW, VW, v_pool != nullptr, n_waves) < 16) n_waves = (n_waves + 1) / 2;
   const int KC = ma_chunk_keys(KW, VW, v_pool != nullptr, n_waves);
   if (KC < 4) return -3;
   MaskedAttentionArgs a;
   a.q_stride = q_stride; a.gate_stride = gate_stride; a.scale = scale; a.cap = cap;
   a.window = window; a.chunk = chunk; a.gate_mode = gate_mode; a.nH = nH; a.nKV = nKV;
   a.KW = KW; a.VW = VW; a.page_size = page_size; a.max_pages = max_pages; a.KC = KC;
-  dim3 grid(T, nKV, (G + MA_MAX_WAVES - 1) / MA_MAX_WAVES);
+  dim3 grid(T, nKV, (G + n_waves - 1) / n_waves);
   const size_t smem = ((size_t)KC * (KW + 1) + (v_pool != nullptr ? (size_t)KC * (VW + 1) : 0)
                        + (size_t)n_waves * (KW + ZF_WAVE) + KC) * sizeof(float);
   if (dtype == ZF_F32)
