@@ -23,6 +23,10 @@ intermediate 25600; 65.5 GB of weights): a 2048-token prefill, then decode at ba
 64 with every request's context just below 8192 tokens; the cache pool is sized for
 64 x 8192 tokens (137 GB).
 
+``--workload fezupel`` and ``--workload lodenex``: shapes of those two designs at layer sizes that
+resemble served models, each beside the dense Qwen3 decoder of equal size (prefill of 2048
+tokens, decode at batch 8), and their kernels alone beside the like kernels of that decoder.
+
 The reference publishes no numbers, so ``vs_baseline`` is null.
 """
 from __future__ import annotations

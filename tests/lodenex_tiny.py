@@ -71,9 +71,9 @@ LX_C = {"architecture": "Lodenex", "vocab": 97, "width": 50, "norm": {"eps": 1e-
 LX_D = {"architecture": "Lodenex", "vocab": 512, "width": 128, "norm": {"eps": 1e-6},
         "embedding": {"scale": 0.25}, "logit_softcap": 20.0,
         "layers": [_attention(4, 2, 64, 64, 48, 0.125, 15.0, 32, 10000.0, _by_wavelength(8.0, 1.0, 4.0, 128), 192),
-                   _latent(4, 32, 32, 32, 64, 64, 40, 0.15, 10000.0, _by_turns(4.0, 64, 32.0, 1.0), 128),
-                   _attention(8, 1, 96, 96, 100, 0.18, 25.0, 32, 500000.0, None, None),
-                   _latent(2, 64, 32, 64, 128, 128, 31, 0.11, 1000.0, _by_turns(16.0, 48, 8.0, 1.0), 64)]}
+                   _latent(4, 32, 32, 32, 64, 64, 44, 0.15, 10000.0, _by_turns(4.0, 64, 24.0, 1.0), 128),
+                   _attention(8, 1, 96, 96, 100, 0.18, 25.0, 32, 250000.0, None, None),
+                   _latent(2, 48, 32, 80, 112, 128, 31, 0.11, 1000.0, _by_turns(16.0, 48, 8.0, 1.0), 64)]}
 
 CONFIGS = {"A": LX_A, "B": LX_B, "C": LX_C, "D": LX_D}
 PAGE_SIZE = {"A": 16, "B": 8, "C": 4, "D": 16}

@@ -270,7 +270,7 @@ CASES = [  # H, G, KW, VW, page, lens, q_lens, cap, window, chunk
     (20, 1, 10, 6, 4, [17, 30], [17, 2], 8.0, 0, 1),
     (6, 2, 8, 12, 16, [150], [150], 2.5, 0, 1000),
     (2, 1, 40, 24, 16, [100, 65, 33], [1, 1, 1], 30.0, 0, 32),
-    (5, 5, 96, 96, 16, [200], [60], 20.0, 40, 0),
+    (5, 5, 96, 96, 16, [200], [60], 18.0, 37, 0),
     (2, 2, 7, 3, 2, [11], [11], 1.5, 3, 4),
 ]
 
@@ -410,10 +410,10 @@ def _run_mfma(pg, qs, q_lens, H, scale, cap=0.0, window=0, chunk=0, sink=None, g
 
 
 MFMA_CASES = [  # H, G, KW, VW, tied, page, lens, q_lens, cap, window, chunk
-    (4, 2, 96, 96, False, 16, [230, 90, 33], [230, 90, 33], 20.0, 0, 120),
+    (6, 3, 96, 96, False, 16, [230, 90, 33], [230, 90, 33], 12.0, 0, 100),
     (8, 8, 64, 64, False, 16, [300, 41], [77, 2], 0.0, 100, 0),
     (32, 1, 128, 128, False, 16, [150], [150], 5.0, 0, 1000),
-    (6, 1, 160, 128, True, 16, [200, 64], [200, 10], 0.0, 40, 0),
+    (5, 1, 160, 128, True, 16, [200, 64], [200, 10], 0.0, 50, 0),
     (3, 1, 96, 64, True, 8, [333], [333], 0.0, 0, 0),
     (16, 1, 192, 128, True, 16, [500], [100], 0.0, 256, 0),
     (12, 4, 128, 128, False, 32, [700], [700], 30.0, 0, 0),
