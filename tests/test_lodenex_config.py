@@ -188,3 +188,19 @@ def test_the_plain_masks_and_the_sink():
     assert out[0, 0, 0] == pytest.approx(1.0 / 3.0) and out[0, 1, 0] == pytest.approx(1.0)
     assert P.tanh_cap(torch.tensor(1000.0), 5.0) == pytest.approx(5.0)
     assert float(P.gelu_erf(torch.tensor(1.0, dtype=torch.float64))) == pytest.approx(0.8413447460685429)
+
+
+def test_command_line_writes_and_inspects_a_model_folder(tmp_path, capsys):
+    from zinfer_amd.cli import main
+    cfg = tmp_path / "config.json"
+    cfg.write_text(json.dumps(lx.LX_B))
+    out = str(tmp_path / "m")
+    assert main(["random-model", str(cfg), out, "--seed", "4", "--dtype", "float32"]) == 0
+    assert main(["inspect-config", out]) == 0
+    text = capsys.readouterr().out
+    assert "architecture: Lodenex" in text and "width: 72" in text and "model_type: lodenex" in text
+    assert text.count("architecture:") == 1
+    assert main(["inspect-weights", out]) == 0
+    text = capsys.readouterr().out
+    assert "tensor l0.mix.dkv.norm: dtype=F32 shape=[32] " in text
+    assert "tensor l0.mix.uk: dtype=F32 shape=[32, 32] " in text and "tensor_count: 50" in text
