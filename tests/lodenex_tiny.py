@@ -49,12 +49,13 @@ LX_A = {"architecture": "Lodenex", "vocab": 211, "width": 48, "norm": {"eps": 1e
                    _attention(2, 1, 16, 8, 11, 0.25, 30.0, 16, 10000.0, None, 36)]}
 
 # a chunk of several pages and one longer than any prompt, a window longer than any prompt;
-# kv heads = query heads; no rule for the latent layer's frequencies; two latent layers in a row
+# kv heads = query heads; no rule for the latent layer's frequencies; two latent layers in a row;
+# a layer whose scores have no cap
 LX_B = {"architecture": "Lodenex", "vocab": 300, "width": 72, "norm": {"eps": 1e-6},
         "embedding": {"scale": 1.0}, "logit_softcap": 30.0,
         "layers": [_latent(2, 16, 8, 12, 40, 32, 1000, 0.2, 10000.0, None, 64),
                    _latent(5, 4, 6, 6, 12, 20, 26, 0.45, 300.0, _by_turns(8.0, 32, 16.0, 2.0), 24),
-                   _attention(3, 3, 16, 16, 40, 0.25, 50.0, 4, 1000.0, _by_wavelength(8.0, 1.0, 4.0, 64), None),
+                   _attention(3, 3, 16, 16, 40, 0.25, None, 4, 1000.0, _by_wavelength(8.0, 1.0, 4.0, 64), None),
                    _attention(6, 2, 8, 12, 1000, 0.4, 2.5, 8, 20.0, _by_wavelength(2.0, 2.0, 8.0, 40), 20)]}
 
 # 20 query heads on one kv head, sizes that are no multiple of 4, a chunk and a window of one

@@ -29,8 +29,6 @@ def by_wavelength(freqs: Tuple[float, ...], factor: float, low: float, high: flo
     """Pairs whose wavelength 2 pi / f is shorter than original / high keep their frequency,
     those longer than original / low turn ``factor`` times slower, and between the two the
     frequency goes in a straight line (in original / wavelength) from the one to the other."""
-    if high == low:
-        raise ConfigError("wavelength scaling needs low != high")
     out = []
     for f in freqs:
         wavelength = 2.0 * math.pi / f
@@ -38,6 +36,8 @@ def by_wavelength(freqs: Tuple[float, ...], factor: float, low: float, high: flo
             out.append(f)
         elif wavelength > original / low:
             out.append(f / factor)
+        elif high == low:              # no range between the two: the one wavelength on the edge
+            out.append(f)
         else:
             t = (original / wavelength - low) / (high - low)
             out.append((1.0 - t) * f / factor + t * f)
